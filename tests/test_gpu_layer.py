@@ -344,6 +344,7 @@ class _RMSNorm:
         (W.RoutingMode("sigmoid", False, "input"), True, None),   # reference mode: rows are copied
         (W.RoutingMode("softmax", True, "output"), False, None),  # rows read through the permutation
         (W.RoutingMode("softmax", True, "output"), False, "fp8"),
+        (W.RoutingMode("softmax", True, "output"), False, "prefill"),  # above 4096 tokens
     ],
 )
 def test_pre_norm_and_residual_in_one_call(gpu_device, dtype, mode, shared, weights):
@@ -354,8 +355,11 @@ def test_pre_norm_and_residual_in_one_call(gpu_device, dtype, mode, shared, weig
     if weights == "fp8" and dtype == "fp32":
         pytest.skip("e4m3 weights go with bf16 activations")
     _say("pre-norm", dtype, mode, shared, weights)
-    # 1300 tokens: normalised inside the router kernel; 300: by the small kernel in front of it
+    # up to 4096 tokens the rows are normalised by a small kernel in front of the router (300, 1300);
+    # above that inside the router kernel (4200)
     tokens = 1300 if shared else 300
+    if weights == "prefill":
+        tokens, weights = 4200, None
     spec = W.small_spec(tokens=tokens, model_dim=128, num_experts=8, top_k=2, inner_dim=192, dtype=dtype,
                         weight_dtype=weights, shared=shared, mode=mode, seed=41)
     wl = W.make_workload_from_spec(spec)

@@ -78,9 +78,13 @@ def test_router_matches_oracle(gpu_device, dtype, tokens, d, e, k, mode, zipf):
     "tokens,d,e,k,with_weight",
     [
         (257, 256, 16, 4, True),    # a last block of one row (normalised by the kernel in front)
-        (1500, 256, 16, 4, True),   # beyond 1024 tokens the MFMA routers normalise on the way
+        (1500, 256, 16, 4, True),   # up to 4096 tokens a small kernel in front normalises the rows
         (1101, 2048, 128, 8, True),
-        (1100, 100, 10, 2, True),   # ... and so does the FMA router
+        (1100, 100, 10, 2, True),
+        (4100, 256, 16, 4, True),   # beyond 4096 tokens the MFMA routers normalise on the way
+        (4133, 128, 8, 2, False),
+        (4133, 100, 10, 2, True),   # ... and so does the FMA router
+        (8192, 512, 128, 8, True),  # the prefill token count
         (64, 2048, 128, 8, True),   # the decode shape
         (100, 96, 24, 3, False),    # no elementwise weight
         (45, 100, 10, 2, True),     # D, E off the 16-byte grid: element-wise path, FMA router
