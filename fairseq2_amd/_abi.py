@@ -15,7 +15,7 @@ from torch import Tensor
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfs2moe.so")
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
@@ -75,6 +75,11 @@ _PROTOTYPES = {
     ),
     "fs2moe_forward_norm_workspace_bytes": (
         c_int64, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32]
+    ),
+    "fs2moe_forward_static_capacity": (c_int64, []),
+    "fs2moe_forward_static": (
+        c_int32,
+        [c_void_p] * 13 + [c_int32] * 12 + [c_void_p, c_void_p],
     ),
     "fs2moe_forward_norm": (
         c_int32,

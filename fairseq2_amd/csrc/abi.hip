@@ -202,3 +202,69 @@ extern "C" int fs2moe_forward_norm(const void* x, const void* norm_weight, float
                       F, F_shared, tile_m, act_dtype, w_dtype, score_fn, renormalize, scale_input,
                       workspace, workspace_bytes, out, stream);
 }
+
+// ---- the whole layer for callers that cannot allocate ----------------------------------------------
+// Every intermediate of fs2moe_forward lives in one array inside the library's own device image, so
+// the call needs no workspace from the caller and never touches an allocator.  Every device the
+// library runs on holds its own copy of the array, at its own address, until the process ends.
+namespace {
+
+static __device__ __align__(256) unsigned char scratch[FS2MOE_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+// Device address of `scratch` on each device, looked up once per device with that device current.
+// Plain word-sized stores of the same value: a race between two first calls is benign.
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// The address of this device's copy of the array (the array's name is only a host-side handle and
+// must never reach a kernel), or null with the error text set.
+void* static_scratch() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fs2moe::set_error("forward_static: cannot identify the current device (%s, device %d)",
+                      hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  void* p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (p != nullptr) return p;
+  e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || p == nullptr) {
+    fs2moe::set_error("forward_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                      hipGetErrorString(e));
+    return nullptr;
+  }
+  __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);
+  return p;
+}
+
+}  // namespace
+
+extern "C" int64_t fs2moe_forward_static_capacity(void) { return FS2MOE_STATIC_SCRATCH_BYTES; }
+
+extern "C" int fs2moe_forward_static(const void* x, const void* residual, const void* router,
+                                     const float* router_bias, const void* w_gate,
+                                     const void* w_up, const void* w_down, const float* s_gate,
+                                     const float* s_up, const float* s_down,
+                                     const void* shared_gate, const void* shared_up,
+                                     const void* shared_down, int32_t T, int32_t D, int32_t E,
+                                     int32_t K, int32_t F, int32_t F_shared, int32_t tile_m,
+                                     int32_t act_dtype, int32_t w_dtype, int32_t score_fn,
+                                     int32_t renormalize, int32_t scale_input, void* out,
+                                     void* stream) {
+  const int64_t need = fs2moe_forward_workspace_bytes(T, D, E, K, F, F_shared, tile_m, act_dtype);
+  FS2_REQUIRE(need >= 0, "forward_static: bad sizes T=%d D=%d E=%d K=%d F=%d F_shared=%d tile_m=%d",
+              T, D, E, K, F, F_shared, tile_m);
+  FS2_REQUIRE(need <= (int64_t)FS2MOE_STATIC_SCRATCH_BYTES,
+              "forward_static: these sizes need %lld bytes of scratch, the built-in array holds "
+              "%lld; use fs2moe_forward with a workspace of the caller's",
+              (long long)need, (long long)FS2MOE_STATIC_SCRATCH_BYTES);
+  void* ws = static_scratch();
+  if (ws == nullptr) return FS2MOE_ERR_LAUNCH;
+  // Every stage writes what it later reads (nothing in the workspace has to start at zero), so the
+  // previous call's contents need no clearing.
+  return fs2moe_forward(x, residual, router, router_bias, w_gate, w_up, w_down, s_gate, s_up,
+                        s_down, shared_gate, shared_up, shared_down, T, D, E, K, F, F_shared,
+                        tile_m, act_dtype, w_dtype, score_fn, renormalize, scale_input, ws,
+                        FS2MOE_STATIC_SCRATCH_BYTES, out, stream);
+}

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FS2MOE_ABI_VERSION 6
+#define FS2MOE_ABI_VERSION 7
 
 /* element types */
 #define FS2MOE_F32 0
@@ -44,6 +44,9 @@ extern "C" {
 /* limits */
 #define FS2MOE_MAX_EXPERTS 256
 #define FS2MOE_MAX_TOP_K 16
+
+/* bytes of the library's built-in scratch array (fs2moe_forward_static) */
+#define FS2MOE_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)
 
 /* error codes */
 #define FS2MOE_OK 0
@@ -224,6 +227,27 @@ int fs2moe_forward_norm(const void* x, const void* norm_weight, float norm_eps,
                         int32_t tile_m, int32_t act_dtype, int32_t w_dtype, int32_t score_fn,
                         int32_t renormalize, int32_t scale_input, void* workspace,
                         int64_t workspace_bytes, void* out, void* stream);
+
+/*
+ * The whole layer without a workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  Same computation and result as fs2moe_forward, bit for bit; the
+ * intermediates live in a FS2MOE_STATIC_SCRATCH_BYTES array inside the library's device image (one
+ * copy per GPU, held until the process ends), and the call makes no allocation of any kind.
+ *   Sizes whose fs2moe_forward_workspace_bytes(...) exceed fs2moe_forward_static_capacity() are
+ *   rejected with FS2MOE_ERR_ARG (decode-sized batches fit; prefill-sized ones do not).
+ *   All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
+ *   streams or threads) race and must be serialised by the caller.
+ */
+int64_t fs2moe_forward_static_capacity(void);
+int fs2moe_forward_static(const void* x, const void* residual, const void* router,
+                          const float* router_bias, const void* w_gate, const void* w_up,
+                          const void* w_down, const float* s_gate, const float* s_up,
+                          const float* s_down, const void* shared_gate, const void* shared_up,
+                          const void* shared_down, int32_t T, int32_t D, int32_t E, int32_t K,
+                          int32_t F, int32_t F_shared, int32_t tile_m, int32_t act_dtype,
+                          int32_t w_dtype, int32_t score_fn, int32_t renormalize,
+                          int32_t scale_input, void* out, void* stream);
 
 #ifdef __cplusplus
 }
