@@ -37,6 +37,9 @@ _PROTOTYPES = {
          c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
          c_void_p],
     ),
+    "fs2moe_cpu_router_select": (
+        c_int32, [c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]
+    ),
     "fs2moe_dispatch_workspace_bytes": (c_int64, [c_int32, c_int32, c_int32]),
     "fs2moe_dispatch": (
         c_int32,
@@ -187,6 +190,21 @@ def router_topk(
     return idx, w, logits
 
 
+def cpu_router_select(logits: Tensor, top_k: int, score_fn: int = SCORE_SIGMOID,
+                      renormalize: bool = False) -> tuple[Tensor, Tensor]:
+    """Host mirror of the device's selection (``fs2moe_cpu_router_select``): from f32 logits on the
+    CPU, the experts (bit for bit what the device selects from the same logits) and their weights."""
+    lib = load()
+    logits = logits.detach().to("cpu", torch.float32).contiguous()
+    t, e = logits.shape
+    idx = torch.empty((t, top_k), dtype=torch.int32)
+    w = torch.empty((t, top_k), dtype=torch.float32)
+    rc = lib.fs2moe_cpu_router_select(logits.data_ptr(), t, e, top_k, score_fn, int(renormalize),
+                                      idx.data_ptr(), w.data_ptr())
+    _check(rc, "fs2moe_cpu_router_select")
+    return idx, w
+
+
 def _router_workspace(lib, x: Tensor, num_experts: int, split: bool) -> tuple[int | None, int]:
     """(pointer, bytes) of a fresh scratch buffer for the router, or (None, 0)."""
     need = lib.fs2moe_router_workspace_bytes(x.shape[0], x.shape[1], num_experts, dtype_code(x.dtype)) if split else 0
@@ -285,6 +303,16 @@ def pack_fp8_weights(q: Tensor, num_experts: int) -> Tensor:
         raise ValueError("fp8 weights need in-features % 64 == 0 and out-features % 16 == 0")
     b = q.view(torch.uint8).view(num_experts, k // 64, 64, n // 16, 16)
     return b.permute(0, 3, 1, 4, 2).contiguous().view(torch.float8_e4m3fn)
+
+
+def unpack_fp8_weights(tiled: Tensor, num_experts: int) -> Tensor:
+    """Inverse of :func:`pack_fp8_weights`: the kernel's ``(E, out/16, in/64, 16, 64)`` tiles back to
+    the reference orientation ``(E*in, out)``."""
+    if tiled.dtype != torch.float8_e4m3fn or tiled.dim() != 5 or tiled.shape[0] != num_experts:
+        raise ValueError("expected float8_e4m3fn tiles of shape (E, out/16, in/64, 16, 64)")
+    e, n16, k64 = tiled.shape[:3]
+    b = tiled.view(torch.uint8).permute(0, 2, 4, 1, 3).contiguous()  # (E, in/64, 64, out/16, 16)
+    return b.view(e * k64 * 64, n16 * 16).view(torch.float8_e4m3fn)
 
 
 def grouped_swiglu(
@@ -402,6 +430,46 @@ def combine(
     return out
 
 
+def check_layer_arguments(x, router, router_bias, w_gate, w_up, w_down, num_experts, f, scales, shared) -> None:
+    """Shapes, dtypes, devices and contiguity of everything ``fs2moe_forward`` takes as a raw pointer:
+    a mismatched tensor would otherwise be read out of bounds or with the wrong layout on the GPU."""
+    e = num_experts
+    if x.dim() != 2 or not x.is_cuda or not x.is_contiguous():
+        raise ValueError("x must be a contiguous (T, D) tensor on the GPU")
+    t, d = x.shape
+    dev = x.device
+
+    def need(name, tensor, shape, dtype):
+        if tensor is None:
+            raise ValueError(f"{name} is missing")
+        if tuple(tensor.shape) != tuple(shape) or tensor.dtype != dtype:
+            raise ValueError(f"{name} must be {tuple(shape)} {dtype}, got {tuple(tensor.shape)} {tensor.dtype}")
+        if tensor.device != dev or not tensor.is_contiguous():
+            raise ValueError(f"{name} must be contiguous and on {dev}")
+
+    need("router", router, (d, e), x.dtype)
+    if router_bias is not None:
+        need("router_bias", router_bias, (e,), torch.float32)
+    if scales is None:
+        need("gate weights", w_gate, (e * d, f), x.dtype)
+        need("up weights", w_up, (e * d, f), x.dtype)
+        need("down weights", w_down, (e * f, d), x.dtype)
+    else:
+        if x.dtype != torch.bfloat16 or d % 64 or f % 64:
+            raise ValueError("fp8 weights need bf16 activations and D, F multiples of 64")
+        need("gate codes", w_gate, (e, f // 16, d // 64, 16, 64), torch.float8_e4m3fn)
+        need("up codes", w_up, (e, f // 16, d // 64, 16, 64), torch.float8_e4m3fn)
+        need("down codes", w_down, (e, d // 16, f // 64, 16, 64), torch.float8_e4m3fn)
+        need("gate scales", scales[0], (e, f), torch.float32)
+        need("up scales", scales[1], (e, f), torch.float32)
+        need("down scales", scales[2], (e, d), torch.float32)
+    if shared is not None:
+        fs = shared[0].shape[0]
+        need("shared gate", shared[0], (fs, d), x.dtype)
+        need("shared up", shared[1], (fs, d), x.dtype)
+        need("shared down", shared[2], (d, fs), x.dtype)
+
+
 def forward(
     x: Tensor,
     router: Tensor,
@@ -437,6 +505,7 @@ def forward(
     else:
         f = w_gate.shape[1] * 16
     f_shared = shared[0].shape[0] if shared is not None else 0
+    check_layer_arguments(x, router, router_bias, w_gate, w_up, w_down, num_experts, f, scales, shared)
     sizes = (t, d, num_experts, top_k, f, f_shared, tile_m, dtype_code(x.dtype))
     need = lib.fs2moe_forward_workspace_bytes(*sizes) if norm is None else lib.fs2moe_forward_norm_workspace_bytes(*sizes)
     if need < 0:

@@ -9,6 +9,9 @@
 // and the top-k is K rounds of: wave-wide maximum of a 32-bit key (an order-preserving image of the
 // f32 logit; NaN ranks above +inf, as torch.topk ranks it), then a ballot of the lanes that hold
 // that key, lowest expert first, so equal logits resolve to the lower expert id.
+#include <cmath>
+#include <cstring>
+
 #include "common.h"
 
 namespace fs2moe {
@@ -973,4 +976,69 @@ extern "C" int fs2moe_router_topk_norm(const void* x, const void* norm_weight, f
   FS2_REQUIRE(norm_eps >= 0.f, "router: norm_eps %g is negative", (double)norm_eps);
   return router_entry(x, norm_weight, norm_eps, xn, router, bias, T, D, E, K, act_dtype, score_fn,
                       renormalize, topk_idx, topk_w, logits, workspace, workspace_bytes, stream);
+}
+
+// ---- host mirror of the selection -------------------------------------------------------------------
+// What select_topk does with a token's logits, on the host: same key, same rounds, same tie rule.
+// Given the logits a device call returned, its indices are the device's bit for bit (also where two
+// logits are closer than the accumulation error of any reference); the weights follow the same
+// formulas in host float arithmetic and agree to rounding.
+namespace {
+inline uint32_t order_key_host(float v) {
+  uint32_t b;
+  memcpy(&b, &v, 4);
+  if (v != v) return 0xffffffffu;
+  if (v == 0.0f) b = 0;
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+inline float order_key_inv_host(uint32_t k) {
+  uint32_t b = k == 0xffffffffu ? 0x7fc00000u : (k & 0x80000000u) ? (k ^ 0x80000000u) : ~k;
+  float v;
+  memcpy(&v, &b, 4);
+  return v;
+}
+}  // namespace
+
+extern "C" int fs2moe_cpu_router_select(const float* logits, int32_t T, int32_t E, int32_t K,
+                                        int32_t score_fn, int32_t renormalize, int32_t* topk_idx,
+                                        float* topk_w) {
+  FS2_REQUIRE(logits && topk_idx && topk_w, "cpu_router_select: null pointer");
+  FS2_REQUIRE(T >= 0 && E >= 1 && E <= FS2MOE_MAX_EXPERTS && K >= 1 && K <= E &&
+                  K <= FS2MOE_MAX_TOP_K,
+              "cpu_router_select: bad sizes T=%d E=%d K=%d", T, E, K);
+  FS2_REQUIRE(score_fn == FS2MOE_SCORE_SIGMOID || score_fn == FS2MOE_SCORE_SOFTMAX,
+              "cpu_router_select: score_fn %d", score_fn);
+  uint32_t key[FS2MOE_MAX_EXPERTS];
+  float val[FS2MOE_MAX_TOP_K], w[FS2MOE_MAX_TOP_K];
+  for (int t = 0; t < T; ++t) {
+    const float* row = logits + (size_t)t * E;
+    for (int e = 0; e < E; ++e) key[e] = order_key_host(row[e]);
+    for (int r = 0; r < K; ++r) {
+      int best = 0;
+      for (int e = 1; e < E; ++e)
+        if (key[e] > key[best]) best = e;  // strict: the lowest expert keeps a tie
+      topk_idx[(size_t)t * K + r] = best;
+      val[r] = order_key_inv_host(key[best]);
+      key[best] = 0u;
+    }
+    if (score_fn == FS2MOE_SCORE_SIGMOID) {
+      float s = 0.f;
+      for (int r = 0; r < K; ++r) {
+        w[r] = 1.0f / (1.0f + expf(-val[r]));
+        s += w[r];
+      }
+      if (renormalize)
+        for (int r = 0; r < K; ++r) w[r] /= s;
+    } else {
+      float s = 0.f;
+      if (renormalize) {
+        for (int r = 0; r < K; ++r) s += expf(val[r] - val[0]);
+      } else {
+        for (int e = 0; e < E; ++e) s += expf(row[e] - val[0]);
+      }
+      for (int r = 0; r < K; ++r) w[r] = expf(val[r] - val[0]) / s;
+    }
+    for (int r = 0; r < K; ++r) topk_w[(size_t)t * K + r] = w[r];
+  }
+  return FS2MOE_OK;
 }

@@ -104,11 +104,40 @@ class GroupedExpertNetwork(ExpertNetwork):
         self.activation = nn.SiLU()
 
     # ---- fp8 (e4m3) weights: derived, non-persistent buffers next to the Parameters ----------------
+    # Stored as integers (codes as uint8, scales as the int32 bit patterns of their f32 values) so
+    # that Module.to(dtype) / .float() / .bfloat16(), which cast every floating-point buffer, leave
+    # them alone; the properties below hand out the typed views the kernels take.
     _FP8_NAMES = ("gate_q", "inner_q", "output_q", "gate_scale", "inner_scale", "output_scale")
 
     @property
     def has_fp8_weights(self) -> bool:
-        return getattr(self, "gate_q", None) is not None
+        return getattr(self, "_gate_q_bits", None) is not None
+
+    def clear_fp8_weights(self) -> None:
+        """Drops the derived e4m3 buffers: the next forward uses the Parameters again."""
+        for name in self._FP8_NAMES:
+            if hasattr(self, f"_{name}_bits"):
+                delattr(self, f"_{name}_bits")
+
+    def _fp8_view(self, name: str) -> Tensor:
+        bits = getattr(self, f"_{name}_bits")
+        want = torch.uint8 if name.endswith("_q") else torch.int32
+        if bits.dtype != want:
+            raise RuntimeError(f"the fp8 buffer {name} was cast to {bits.dtype}; quantise again")
+        return bits.view(torch.float8_e4m3fn if name.endswith("_q") else torch.float32)
+
+    gate_q = property(lambda self: self._fp8_view("gate_q"))
+    inner_q = property(lambda self: self._fp8_view("inner_q"))
+    output_q = property(lambda self: self._fp8_view("output_q"))
+    gate_scale = property(lambda self: self._fp8_view("gate_scale"))
+    inner_scale = property(lambda self: self._fp8_view("inner_scale"))
+    output_scale = property(lambda self: self._fp8_view("output_scale"))
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        # new Parameters make the derived codes stale
+        if any(k.startswith(prefix) for k in state_dict):
+            self.clear_fp8_weights()
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     def load_fp8_weights(self, gate_q, gate_scale, inner_q, inner_scale, output_q, output_scale):
         """Installs pre-quantised weights.  Codes are ``float8_e4m3fn`` in the reference orientation
@@ -133,7 +162,8 @@ class GroupedExpertNetwork(ExpertNetwork):
             (codes(gate_q, d, f), codes(inner_q, d, f), codes(output_q, f, d),
              scale(gate_scale, f), scale(inner_scale, f), scale(output_scale, d)),
         ):
-            self.register_buffer(name, val, persistent=False)
+            bits = val.view(torch.uint8) if name.endswith("_q") else val.view(torch.int32)
+            self.register_buffer(f"_{name}_bits", bits, persistent=False)
 
     @torch.no_grad()
     def quantize_fp8_(self) -> None:
@@ -188,9 +218,22 @@ class GroupedExpertNetwork(ExpertNetwork):
         e, n, d = x.shape
         if e != self.num_local_experts or d != self.model_dim:
             raise ValueError(f"expected ({self.num_local_experts}, *, {self.model_dim}), got {tuple(x.shape)}")
-        counts = torch.full((e,), n, dtype=torch.int32, device=x.device)
-        offsets = torch.arange(e + 1, dtype=torch.int32, device=x.device) * n
+        counts, offsets = self._uniform_groups(n, x.device)
         return self.forward_rows(x.reshape(e * n, d).contiguous(), counts, offsets).view(e, n, d)
+
+    def _uniform_groups(self, n: int, device: torch.device) -> tuple[Tensor, Tensor]:
+        """counts / offsets of ``n`` rows for every expert, built once per (n, device) so that the
+        call itself launches nothing but the expert kernels (and records cleanly into a HIP graph)."""
+        cache = self.__dict__.setdefault("_uniform_cache", {})
+        key = (n, str(device))
+        if key not in cache:
+            e = self.num_local_experts
+            cache.clear()
+            cache[key] = (
+                torch.full((e,), n, dtype=torch.int32, device=device),
+                torch.arange(e + 1, dtype=torch.int32, device=device) * n,
+            )
+        return cache[key]
 
 
 class _Projection(Module):
@@ -347,6 +390,11 @@ class MoE(FeedForwardNetwork):
     def forward(self, seqs: Tensor, *, residual: Tensor | None = None, norm=None) -> Tensor:
         """``seqs``: ``(*, dim)`` -> ``(*, dim)``, same dtype.
 
+        Under ``torch.autocast("cuda", dtype)`` (the reference trainer wraps the model in it,
+        ``trainer.py:650-656``) ``seqs`` is cast to the autocast dtype when the module's parameters
+        are held in it, and the result comes back in that dtype, as the reference's matrix products
+        would leave it; parameters of another dtype are not cast behind the caller's back.
+
         ``residual`` (keyword-only extension, same shape and dtype as ``seqs``): returns
         ``residual + layer(seqs)`` from one accumulation, i.e. the feed-forward half of a pre-norm
         decoder layer (``models/transformer_lm/decoder_layer.py:188-204``) without the separate
@@ -358,6 +406,9 @@ class MoE(FeedForwardNetwork):
         normalised inside the router kernel instead of by a pass of their own, so that
         ``layer(seqs, residual=seqs, norm=layer_norm)`` is the whole of ``_forward_ffn``
         (``decoder_layer.py:187-204``) for a pre-norm layer without dropout."""
+        seqs = self._autocast(seqs)
+        if residual is not None:
+            residual = self._autocast(residual)
         x = self._checked_rows(seqs)
         norm_args = self._norm_args(norm, x)
         res = None
@@ -373,6 +424,13 @@ class MoE(FeedForwardNetwork):
         if type(ex) is GroupedExpertNetwork and (se is None or type(se) is GLUFeedForwardNetwork):
             return self._single_call(x, res, norm_args).view(seqs.shape)
         return self._stages(x, res, norm_args)[0].view(seqs.shape)
+
+    def _autocast(self, t: Tensor) -> Tensor:
+        if t.is_cuda and torch.is_autocast_enabled("cuda"):
+            dt = torch.get_autocast_dtype("cuda")
+            if t.is_floating_point() and t.dtype != dt and self.router.dtype == dt:
+                return t.to(dt)
+        return t
 
     @staticmethod
     def _norm_args(norm, x: Tensor) -> tuple[Tensor | None, float] | None:
@@ -475,7 +533,11 @@ class MoE(FeedForwardNetwork):
         _require_device(seqs)
         _require_forward_only(seqs, *self.parameters())
         if seqs.dtype != self.router.dtype:
-            raise TypeError(f"seqs is {seqs.dtype} but the module holds {self.router.dtype} parameters")
+            hint = ""
+            if torch.is_autocast_enabled("cuda"):
+                hint = (f" (autocast to {torch.get_autocast_dtype('cuda')} is on: hold the module's "
+                        "parameters in that dtype)")
+            raise TypeError(f"seqs is {seqs.dtype} but the module holds {self.router.dtype} parameters{hint}")
         dim = seqs.shape[-1]
         if dim != self.router.shape[0]:
             raise ValueError(f"last dimension of seqs is {dim}, expected {self.router.shape[0]}")

@@ -99,6 +99,19 @@ int fs2moe_router_topk_norm(const void* x, const void* norm_weight, float norm_e
                             int64_t workspace_bytes, void* stream);
 
 /*
+ * Host mirror of the router's selection: from a token's logits (HOST memory, bias included, e.g. the
+ * `logits` output of fs2moe_router_topk copied back) the K experts and their weights, by the rule the
+ * device applies (descending; ties to the lower expert id; NaN highest; -0 = +0).  The indices equal
+ * the device's bit for bit, near-ties included; the weights agree to float rounding.  Runs on the
+ * CPU and touches no GPU: it is what lets a test or an integrator verify the routing exactly where
+ * two logits are closer than the accumulation error of any reference matmul.
+ * Replaces torch.topk and the score function of moe.py:113-127 on given logits.
+ *   logits [T, E] f32 (host)     topk_idx [T, K] int32 (host, out)     topk_w [T, K] f32 (host, out)
+ */
+int fs2moe_cpu_router_select(const float* logits, int32_t T, int32_t E, int32_t K, int32_t score_fn,
+                             int32_t renormalize, int32_t* topk_idx, float* topk_w);
+
+/*
  * Bytes of device scratch fs2moe_dispatch needs (per-block histograms and ranks).
  */
 int64_t fs2moe_dispatch_workspace_bytes(int32_t T, int32_t K, int32_t E);

@@ -11,11 +11,22 @@ from oracle import moe_oracle as O
 
 TORCH_DTYPE = {"fp32": torch.float32, "bf16": torch.bfloat16}
 
-# Output tolerance: |y - ref| <= atol + rtol * |ref| with atol tied to the output RMS (outputs are
-# zero-mean sums, so a pure relative test is ill-conditioned near zero).
-#   bf16: rtol 2e-2 (the stated bound for bf16), atol 2e-2 * rms
-#   fp32: rtol 1e-4, atol 1e-4 * rms  (f32 MFMA accumulation order differs from the CPU BLAS)
-TOL = {"bf16": (2e-2, 2e-2), "fp32": (1e-4, 1e-4)}
+# Output tolerance, two statements per comparison.
+#   element-wise: |y - ref| <= atol + rtol * |ref| with atol tied to the output RMS (outputs are
+#     zero-mean sums, so a pure relative test is ill-conditioned near zero);
+#   overall: rms(y - ref) <= RMS_TOL * rms(ref).
+# bf16: rtol 2e-2 (the stated bound for bf16).  Every term of an output element passes three bf16
+#   roundings (the scaled or plain input row, h, the expert's output row) and the sum a fourth; each
+#   is at most 2^-9 relative, so the error of an element behaves like a zero-mean variable of
+#   standard deviation sigma ~ 2^-9 * rms(ref) * c, c between 1 and 2 with the SiLU gate's slope
+#   (0.37 % of rms(ref) in the CPU emulation of the rounding points at K = 16 with scaled inputs,
+#   tests/test_oracle_pins.py).  The largest of N such errors is about sqrt(2 ln N) sigma: 5.3 sigma
+#   = 2 % of rms(ref) for the 5.6e5 elements of a 1100 x 512 output, so atol = 2 % sits AT the expected
+#   maximum (a seeded case did land at 1.03 of it); atol = 4e-2 * rms is 10 sigma.  The overall
+#   statement, RMS_TOL = 1e-2, is the sharp one: 2.7 sigma-units above the emulation's 0.37 %.
+# fp32: rtol 1e-4, atol 1e-4 * rms, RMS_TOL 2e-5 (f32 MFMA accumulation order differs from the CPU's).
+TOL = {"bf16": (2e-2, 4e-2), "fp32": (1e-4, 1e-4)}
+RMS_TOL = {"bf16": 1e-2, "fp32": 2e-5}
 
 
 def oracle_routing(wl: W.Workload):
@@ -46,13 +57,45 @@ def assert_output_close(got: torch.Tensor, ref: torch.Tensor, dtype: str, what: 
     atol = atol_rel * rms
     err = (got - ref).abs()
     bound = atol + rtol * ref.abs()
-    worst = float((err / bound).max())
+    worst = float((err / bound).max()) if err.numel() else 0.0
     assert torch.isfinite(got).all(), f"{what}: non-finite values"
     assert worst <= 1.0, (
         f"{what}: max err/bound = {worst:.3f} (max abs err {float(err.max()):.3e}, rms {rms:.3e}, "
         f"rtol {rtol}, atol {atol:.3e})"
     )
+    err_rms = float(err.pow(2).mean().sqrt()) if err.numel() else 0.0
+    assert err_rms <= RMS_TOL[dtype] * rms or rms == 0.0, (
+        f"{what}: rms error {err_rms:.3e} above {RMS_TOL[dtype]} of the output rms {rms:.3e}"
+    )
+    print(f"  {what}: worst err/bound {worst:.3f}, rms err / rms {err_rms / rms if rms else 0.0:.2e}", flush=True)
     return worst
+
+
+def emulate_device_rounding(wl: W.Workload, idx, w, residual=None):
+    """The layer evaluated on the CPU in f32 with a bf16 rounding at every point where the device
+    rounds (the scaled input row in the reference mode, h, the expert's output row, the final sum in
+    ascending expert id): what the HIP path computes up to the order of f32 additions inside a dot
+    product.  bf16 workloads without a shared expert only.  Returns the (T, D) result as f32."""
+    s = wl.spec
+    assert s.dtype == "bf16" and not s.shared
+    t, d, e, f = s.num_tokens, s.model_dim, s.num_experts, s.inner_dim
+    bf = lambda v: v.to(torch.bfloat16).float()  # noqa: E731
+    x = wl.x.reshape(t, d).float()
+    gate, up, down = wl.gate.float().view(e, d, f), wl.up.float().view(e, d, f), wl.down.float().view(e, f, d)
+    w32 = w.float()
+    out = torch.zeros(t, d) if residual is None else residual.reshape(t, d).float().clone()
+    scale_in = s.mode.scale_on == "input"
+    for ex in range(e):
+        sel = idx == ex
+        tok = sel.any(dim=1).nonzero().squeeze(1)
+        if tok.numel() == 0:
+            continue
+        we = (w32 * sel).sum(dim=1)[tok]
+        xe = bf(x[tok] * we[:, None]) if scale_in else x[tok]
+        h = bf(torch.nn.functional.silu(xe @ gate[ex]) * (xe @ up[ex]))
+        ye = bf(h @ down[ex])
+        out[tok] += ye if scale_in else ye * we[:, None]
+    return bf(out)
 
 
 def assert_routing_equal(idx_gpu, disp, r: O.Routing, what: str = ""):

@@ -9,6 +9,7 @@ import torch
 
 from fairseq2_amd import _abi
 from fairseq2_amd import moe as M
+from oracle import moe_oracle as O
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "fs2moe.h")
@@ -228,3 +229,72 @@ def test_norm_argument_is_validated_before_anything_runs():
     # a weight must live on the GPU like everything else (no CPU fallback)
     with pytest.raises(RuntimeError, match="GPU only"):
         M.MoE._norm_args(Norm(torch.ones(64), None, 1e-5, (64,)), x)
+
+
+def test_host_mirror_of_the_selection_matches_the_oracle(lib):
+    """fs2moe_cpu_router_select on the CPU: the oracle's ordered top-k (ties to the lower expert,
+    NaN highest, -0 = +0, -inf selectable last) and weights in all four score modes."""
+    g = torch.Generator().manual_seed(2)
+    logits = torch.randn(400, 24, generator=g)
+    logits[0] = 0.0  # all equal: experts 0..K-1
+    logits[1, 3] = float("nan")
+    logits[2, 5] = float("inf")
+    logits[3, :4] = 1.0
+    logits[4, 7] = -0.0
+    logits[4, 2] = 0.0
+    logits[5, 6:] = float("-inf")
+    logits[6] = torch.round(logits[6] * 2) / 2  # many exact ties
+    for k in (1, 6, 16):
+        for score_fn, renorm, name in ((0, False, "sigmoid"), (0, True, "sigmoid"), (1, False, "softmax"), (1, True, "softmax")):
+            idx, w = _abi.cpu_router_select(logits, k, score_fn, renorm)
+            ref = O.topk_lowest_index(logits.double(), k)
+            assert torch.equal(idx.long(), ref), (k, name, renorm)
+            wr = O.combine_weights(logits.double(), ref, name, renorm)
+            ok = ~torch.isnan(wr)
+            assert torch.allclose(w.double()[ok], wr[ok], rtol=2e-6, atol=1e-7), (k, name, renorm)
+            assert bool(torch.isnan(w.double()[~ok]).all())
+    # argument errors
+    rc = lib.fs2moe_cpu_router_select(logits.data_ptr(), 4, 24, 25, 0, 0, logits.data_ptr(), logits.data_ptr())
+    assert rc == -1
+
+
+def test_fp8_buffers_follow_the_parameters():
+    """The e4m3 codes and scales are derived from the Parameters: loading new Parameters drops them,
+    clear_fp8_weights() drops them, and Module.to(dtype), which casts floating-point buffers, cannot
+    touch them (they are stored as integers and viewed at call time)."""
+    m = M.MoE(64, 64, False, 4, 1.0, 2, inner_dim_scale=1.0, auto_scale=False)
+    g = torch.Generator().manual_seed(0)
+    with torch.no_grad():
+        for p in m.parameters():
+            p.copy_(0.1 * torch.randn(p.shape, generator=g))
+    ex = m.experts
+    assert not ex.has_fp8_weights
+    ex.quantize_fp8_()
+    assert ex.has_fp8_weights
+    assert ex.gate_q.dtype == torch.float8_e4m3fn and ex.gate_q.shape == (4, 64 // 16, 64 // 64, 16, 64)
+    assert ex.output_scale.dtype == torch.float32 and ex.output_scale.shape == (4, 64)
+    codes = ex.gate_q.view(torch.uint8).clone()
+    m.to(torch.bfloat16)
+    assert ex.has_fp8_weights and ex.gate_q.dtype == torch.float8_e4m3fn
+    assert torch.equal(ex.gate_q.view(torch.uint8), codes)
+    assert ex.gate_scale.dtype == torch.float32
+    m.float()
+    assert torch.equal(ex.gate_q.view(torch.uint8), codes)
+    assert "gate_q" not in m.state_dict() and not any("bits" in k for k in m.state_dict())
+    m.load_state_dict(m.state_dict())
+    assert not ex.has_fp8_weights, "new Parameters make the derived codes stale"
+    ex.quantize_fp8_()
+    ex.clear_fp8_weights()
+    assert not ex.has_fp8_weights
+    with pytest.raises(AttributeError):
+        ex.gate_q
+
+
+def test_fp8_tile_packing_round_trip():
+    g = torch.Generator().manual_seed(1)
+    q = (50 * torch.randn(3 * 128, 80, generator=g)).to(torch.float8_e4m3fn)
+    tiled = _abi.pack_fp8_weights(q, 3)
+    assert tiled.shape == (3, 5, 2, 16, 64)
+    # tile (e, c, k) holds channels 16 c .. 16 c + 15 (rows) x input features 64 k .. 64 k + 63
+    assert tiled.view(torch.uint8)[1, 2, 1, 3, 5] == q.view(torch.uint8)[1 * 128 + 64 + 5, 2 * 16 + 3]
+    assert torch.equal(_abi.unpack_fp8_weights(tiled, 3).view(torch.uint8), q.view(torch.uint8))

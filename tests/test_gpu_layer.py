@@ -183,11 +183,11 @@ def test_qwen3_30b_a3b_shape(gpu_device):
 
 
 def test_mixtral_8x7b_shape(gpu_device):
-    _full_size_case("mixtral_8x7b", gpu_device, sample=48)
+    _full_size_case("mixtral_8x7b", gpu_device, sample=256)
 
 
 def test_llama4_scout_shape(gpu_device):
-    _full_size_case("llama4_scout", gpu_device, sample=48)
+    _full_size_case("llama4_scout", gpu_device, sample=256)
 
 
 def test_qwen3_decode_fp8_shape(gpu_device):
@@ -446,3 +446,226 @@ def test_module_under_torch_compile(gpu_device, case):
         again = compiled(x)
     torch.cuda.synchronize()
     assert torch.equal(got, want) and torch.equal(again, want)
+
+
+# --------------------------------------------------------------------------- interface rows
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_grouped_expert_network_in_the_reference_calling_convention(gpu_device, dtype):
+    """``GroupedExpertNetwork.forward((E, n, D))`` is how the reference calls its experts
+    (experts.py:201-213): every expert gets the same number of rows.  Each expert against the oracle's
+    textbook SwiGLU in f64; the call launches nothing but the expert kernels, so it records into a HIP
+    graph, and the replays give the eager bits."""
+    from fairseq2_amd.moe import GroupedExpertNetwork
+
+    _say("GroupedExpertNetwork.forward", dtype)
+    e, n, d, f = 6, 37, 128, 192
+    td = TORCH_DTYPE[dtype]
+    g = torch.Generator().manual_seed(17)
+    net = GroupedExpertNetwork(e, d, f, device=gpu_device, dtype=td).requires_grad_(False)
+    wg = (0.05 * torch.randn(e * d, f, generator=g)).to(td)
+    wu = (0.05 * torch.randn(e * d, f, generator=g)).to(td)
+    wd = (0.05 * torch.randn(e * f, d, generator=g)).to(td)
+    net.load_state_dict({"gate_proj": wg, "inner_proj": wu, "output_proj": wd})
+    x = torch.randn(e, n, d, generator=g).to(td)
+    xd = x.to(gpu_device)
+    with torch.no_grad():
+        y = net(xd)
+        y2 = net(xd)
+    torch.cuda.synchronize()
+    assert y.shape == (e, n, d) and y.dtype == td and torch.equal(y, y2)
+    for ex in range(e):
+        want = O.glu_expert(x[ex].double(), wg.double().view(e, d, f)[ex], wu.double().view(e, d, f)[ex],
+                            wd.double().view(e, f, d)[ex])
+        assert_output_close(y[ex], want, dtype, f"expert {ex}")
+    with pytest.raises(ValueError):
+        net(xd[:, :, : d // 2])
+    # graph-clean: counts and offsets are built once, the call is kernels only
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        net(xd)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph), torch.no_grad():
+        yg = net(xd)
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(yg, y)
+        with torch.no_grad():
+            net(xd)  # eager work between replays
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_llama4_checkpoint_names_load_and_run(gpu_device, fp8):
+    """A Meta-format Llama-4 state dict (llama4/interop.py:126-136) goes through
+    ``load_llama4_moe_layer`` into the module on the GPU, optionally packed to e4m3, and the forward
+    pass is the oracle's on the same tensors (on the de-quantised ones with fp8)."""
+    from fairseq2_amd import MoE
+    from fairseq2_amd.checkpoint import load_llama4_moe_layer
+
+    _say("llama4 checkpoint", fp8)
+    d, e, f, t = 128, 8, 192, 200
+    g = torch.Generator().manual_seed(23)
+    r = lambda *s: (0.05 * torch.randn(*s, generator=g)).to(torch.bfloat16)  # noqa: E731
+    p = "layers.2.feed_forward."
+    sd = {
+        "tok_embeddings.weight": r(10, d),
+        p + "router_DE": (4.0 * r(d, e)),
+        p + "experts.moe_w_in_eD_F": r(e * d, f),
+        p + "experts.moe_w_swiglu_eD_F": r(e * d, f),
+        p + "experts.moe_w_out_eF_D": r(e * f, d),
+        p + "w_in_shared_FD.weight": r(f, d),
+        p + "w_swiglu_FD.weight": r(f, d),
+        p + "w_out_shared_DF.weight": r(d, f),
+        p + "running_gate_stats_3E": r(3, e),
+        p + "experts._extra_state": r(1),
+    }
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        m = MoE(d, f, True, e, 1.0, 1, inner_dim_scale=1.0, auto_scale=False)
+    finally:
+        torch.set_default_dtype(prev)
+    m = m.to(gpu_device).requires_grad_(False)
+    load_llama4_moe_layer(m, sd, 2, fp8=fp8)
+    assert m.experts.has_fp8_weights == fp8
+    x = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
+    with torch.no_grad():
+        out, gi, gw, disp = m.forward_with_routing(x.to(gpu_device))
+        again = m(x.to(gpu_device))
+    torch.cuda.synchronize()
+    assert torch.equal(out, again)
+    gate, up, down = (sd[p + n].float() for n in ("experts.moe_w_in_eD_F", "experts.moe_w_swiglu_eD_F",
+                                                  "experts.moe_w_out_eF_D"))
+    if fp8:
+        # the codes the module holds (quantised on the device: where w / scale lands on a rounding
+        # boundary torch's device cast may pick the other neighbour than the CPU's, and both are
+        # valid e4m3 images of the weight), de-quantised
+        ex = m.experts
+        gate, up, down = (
+            W.dequantize_fp8_per_channel(_abi.unpack_fp8_weights(q, e).cpu(), s.cpu())
+            for q, s in ((ex.gate_q, ex.gate_scale), (ex.inner_q, ex.inner_scale), (ex.output_q, ex.output_scale))
+        )
+        for deq_w, name in ((gate, "experts.moe_w_in_eD_F"), (down, "experts.moe_w_out_eF_D")):
+            # ... and they ARE images of the checkpoint's weights: within one e4m3 step (2^-3 relative,
+            # 2^-9 * 448 * scale below the normal range), most within half of one
+            rel = (deq_w - sd[p + name].float()).abs() / sd[p + name].float().abs().clamp_min(1e-3)
+            assert float(rel.max()) <= 0.126 and float(rel.mean()) < 0.03
+    shared = tuple(sd[p + n].double() for n in ("w_in_shared_FD.weight", "w_swiglu_FD.weight", "w_out_shared_DF.weight"))
+    logits = O.router_logits(x.reshape(-1, d).double(), sd[p + "router_DE"].double(), None)
+    idx = O.topk_lowest_index(logits, 1)
+    ref = O.ref_sparse_forward(x.double(), sd[p + "router_DE"].double(), gate.double(), up.double(), down.double(), 1,
+                               shared=shared, tile_m=m.tile_m, topk_idx=idx)
+    assert_routing_equal(gi, disp, ref.routing, "llama4 checkpoint")
+    assert_output_close(out, ref.out, "bf16", "llama4 checkpoint")
+    # loading plain weights afterwards drops the derived e4m3 buffers
+    if fp8:
+        load_llama4_moe_layer(m, sd, 2, fp8=False)
+        assert not m.experts.has_fp8_weights
+
+
+def test_scout_constructor_arguments_of_the_reference_factory(gpu_device):
+    """The module as the Llama-4 factory constructs it for Scout (llama4/factory.py:123-135:
+    inner dim 4 * 5120 * 1.2 = 24576, scale 2/3, auto-scaled by capacity + shared, rounded up to a
+    multiple of 2048) has the 8192-wide experts of the workload, and computes the same as the module
+    built with the inner dim given outright."""
+    from fairseq2_amd import MoE
+
+    _say("scout ctor")
+    wl = W.make_workload("llama4_scout")
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        m = MoE(5120, 24576, True, 16, 1.0, 1, inner_dim_to_multiple=2048)
+    finally:
+        torch.set_default_dtype(prev)
+    assert m.experts.inner_dim == 8192 and m.shared_expert.gate_proj.weight.shape == (8192, 5120)
+    direct = build_module(wl, gpu_device)
+    m.load_state_dict(direct.state_dict(), strict=True)
+    m = m.to(gpu_device).requires_grad_(False).eval()
+    x = wl.x.to(torch.bfloat16).to(gpu_device)[:, :512]
+    with torch.no_grad():
+        assert torch.equal(m(x), direct(x))
+
+
+def test_autocast_is_honoured(gpu_device):
+    """Under torch.autocast (trainer.py:650-656) an f32 input is cast to the autocast dtype when the
+    module holds its parameters in it; the result comes back in that dtype and equals the call on
+    the cast input.  Parameters of another dtype are not cast silently."""
+    _say("autocast")
+    wl = W.make_workload_from_spec(W.small_spec(tokens=64, model_dim=128, num_experts=8, top_k=2, inner_dim=64,
+                                                dtype="bf16", seed=3))
+    m = build_module(wl, gpu_device)
+    x32 = wl.x.float().to(gpu_device)
+    with torch.no_grad():
+        want = m(x32.to(torch.bfloat16))
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got = m(x32)
+            got_res = m(x32, residual=x32)
+        assert got.dtype == torch.bfloat16 and torch.equal(got, want)
+        assert torch.equal(got_res, m(x32.to(torch.bfloat16), residual=x32.to(torch.bfloat16)))
+        with pytest.raises(TypeError, match="parameters"):
+            m(x32)  # no autocast: dtype mismatch is an error
+        wl32 = W.make_workload_from_spec(W.small_spec(tokens=64, model_dim=128, num_experts=8, top_k=2,
+                                                      inner_dim=64, dtype="fp32", seed=3))
+        m32 = build_module(wl32, gpu_device)
+        with torch.autocast("cuda", dtype=torch.bfloat16), pytest.raises(TypeError, match="autocast"):
+            m32(x32.to(torch.bfloat16))
+
+
+def test_reference_arithmetic_in_bf16(gpu_device):
+    """The reference run in bf16 rounds the logits to bf16 before torch.topk and the sigmoid, keeps the
+    scores in bf16 and accumulates scatter_add_ in bf16 (moe.py:109-150 on bf16 tensors).  The device
+    keeps f32 logits and weights and rounds the output once: a deliberate refinement.  Its selection
+    must still be a valid top-k of the bf16-rounded logits (it resolves their ties by the f32 values),
+    and its output must agree with the reference's own bf16 result within the bf16 bound."""
+    _say("reference arithmetic in bf16")
+    spec = W.small_spec(tokens=200, model_dim=128, num_experts=8, top_k=2, inner_dim=96, dtype="bf16", seed=77)
+    wl = W.make_workload_from_spec(spec)
+    m, x, out, gi, gw, disp = _run(wl, gpu_device)
+    b = lambda t_: t_.to(torch.bfloat16)  # noqa: E731
+    logits_bf16 = (b(wl.x).reshape(-1, 128) @ b(wl.router)).float()
+    chosen = torch.gather(logits_bf16, 1, gi.cpu().long())
+    rest = logits_bf16.scatter(1, gi.cpu().long(), float("-inf")).max(dim=1).values
+    assert bool((chosen.min(dim=1).values >= rest).all()), "not a top-k of the bf16-rounded logits"
+    assert bool((chosen[:, :-1] >= chosen[:, 1:]).all())
+    dense_bf16 = O.ref_dense_forward(b(wl.x), b(wl.router), b(wl.gate), b(wl.up), b(wl.down), 2)
+    # where both selections agree (every token here unless a bf16 tie was resolved the other way)
+    ref_idx = torch.topk(b(wl.x).reshape(-1, 128) @ b(wl.router), 2, dim=1).indices
+    same = (torch.sort(ref_idx, dim=1).values == torch.sort(gi.cpu().long(), dim=1).values).all(dim=1)
+    assert float(same.float().mean()) > 0.9
+    got = out.reshape(-1, 128).cpu()[same]
+    assert_output_close(got, dense_bf16.reshape(-1, 128)[same].double(), "bf16", "vs the reference in bf16")
+
+
+def test_layer_arguments_are_validated_before_the_gpu_reads_them(gpu_device):
+    """fs2moe_forward takes raw pointers: the binding refuses tensors whose shape, dtype or device
+    does not match the sizes, instead of letting a kernel read out of bounds."""
+    _say("argument validation")
+    wl = W.make_workload_from_spec(W.small_spec(tokens=32, model_dim=128, num_experts=8, top_k=2, inner_dim=64,
+                                                dtype="bf16", seed=5))
+    m = build_module(wl, gpu_device)
+    ex = m.experts
+    x = wl.x.to(torch.bfloat16).to(gpu_device).reshape(-1, 128)
+    w = (ex.gate_proj.detach(), ex.inner_proj.detach(), ex.output_proj.detach())
+    good = _abi.forward(x, m.router.detach(), None, *w, 8, 2)
+    assert good.shape == x.shape
+    with pytest.raises(ValueError, match="router"):
+        _abi.forward(x, m.router.detach()[:, :4].contiguous(), None, *w, 8, 2)
+    with pytest.raises(ValueError, match="router"):
+        _abi.forward(x, m.router.detach().float(), None, *w, 8, 2)
+    with pytest.raises(ValueError, match="gate weights"):
+        _abi.forward(x, m.router.detach(), None, w[0][:-8].contiguous(), w[1], w[2], 8, 2)
+    with pytest.raises(ValueError, match="up weights"):
+        _abi.forward(x, m.router.detach(), None, w[0], w[1].cpu(), w[2], 8, 2)
+    with pytest.raises(ValueError, match="router_bias"):
+        _abi.forward(x, m.router.detach(), torch.zeros(8, dtype=torch.bfloat16, device=gpu_device), *w, 8, 2)
+    with pytest.raises(ValueError, match="shared"):
+        _abi.forward(x, m.router.detach(), None, *w, 8, 2, shared=(w[0], w[0], w[0]))
+    # an fp8 module whose buffers were cast by .to(dtype) keeps its codes (they are integer buffers)
+    ex.quantize_fp8_()
+    m.to(torch.bfloat16)
+    assert ex.gate_q.dtype == torch.float8_e4m3fn and ex.gate_scale.dtype == torch.float32
+    with torch.no_grad():
+        m(x)

@@ -444,3 +444,65 @@ def test_rms_norm_vs_library_routine(dtype):
         xf = x.float()
         twice = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).to(dtype) * w
         assert not torch.equal(twice, want)
+
+
+def test_sigmoid_renormalised_weights_closed_form():
+    """combine_weights(sigmoid, renormalize=True): sigma(l_e) / sum over the selected of sigma(l_j).
+    Closed forms: equal logits give 1/K each whatever their value; logits (0, +inf-ish) give
+    (1/3, 2/3) since sigma(0) = 1/2 and sigma(40) = 1; the weights of a token sum to one; scaling all
+    selected sigmoids by a common factor (logit pairs (a, b) with sigma(a) = 2 sigma(b)) gives 2/3, 1/3."""
+    k = 3
+    logits = torch.tensor([[1.7, 1.7, 1.7, -5.0], [-2.0, -2.0, -2.0, -9.0]], dtype=torch.float64)
+    idx = O.topk_lowest_index(logits, k)
+    w = O.combine_weights(logits, idx, "sigmoid", True)
+    assert torch.allclose(w, torch.full((2, k), 1.0 / 3.0, dtype=torch.float64), atol=1e-15)
+    logits = torch.tensor([[0.0, 40.0, -50.0]], dtype=torch.float64)
+    idx = O.topk_lowest_index(logits, 2)  # descending: expert 1, then expert 0
+    w = O.combine_weights(logits, idx, "sigmoid", True)
+    assert idx.tolist() == [[1, 0]]
+    assert torch.allclose(w, torch.tensor([[2.0 / 3.0, 1.0 / 3.0]], dtype=torch.float64), atol=1e-12)
+    # sigma(a) = 2 sigma(b) with sigma(b) = 0.3: a = logit(0.6), b = logit(0.3)
+    a, b = math.log(0.6 / 0.4), math.log(0.3 / 0.7)
+    logits = torch.tensor([[b, -30.0, a]], dtype=torch.float64)
+    idx = O.topk_lowest_index(logits, 2)
+    w = O.combine_weights(logits, idx, "sigmoid", True)
+    assert idx.tolist() == [[2, 0]]
+    assert torch.allclose(w, torch.tensor([[2.0 / 3.0, 1.0 / 3.0]], dtype=torch.float64), atol=1e-12)
+    # random logits: rows sum to one and the ratios are the ratios of the plain sigmoids
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(50, 9, generator=g, dtype=torch.float64)
+    idx = O.topk_lowest_index(logits, 4)
+    w = O.combine_weights(logits, idx, "sigmoid", True)
+    plain = O.combine_weights(logits, idx, "sigmoid", False)
+    assert torch.allclose(w.sum(dim=1), torch.ones(50, dtype=torch.float64), atol=1e-14)
+    assert torch.allclose(w * plain[:, :1], plain * w[:, :1], atol=1e-15)
+    # not renormalised, for contrast: the plain sigmoids, which do not sum to one
+    assert torch.allclose(plain, torch.sigmoid(torch.gather(logits, 1, idx)), atol=0)
+
+
+def test_bf16_rounding_budget_of_the_device_pipeline():
+    """The error budget behind the bf16 tolerance (tests/_util.py): the layer evaluated in f32 with a
+    bf16 rounding wherever the device rounds, against the f64 oracle, in the configuration with the
+    most roundings per output element (every one of 16 experts selected, scaled input rows).  The
+    overall error is a few tenths of a percent of the output's rms, well inside RMS_TOL, and every
+    element is inside the element-wise bound with room to spare (the largest errors sit on the largest
+    elements, where the final rounding alone is 2^-9 of the value: they are what rtol is for)."""
+    from fairseq2_amd import workloads as W
+    from tests._util import RMS_TOL, TOL, emulate_device_rounding, oracle_forward, oracle_routing
+
+    spec = W.small_spec(tokens=300, model_dim=256, num_experts=16, top_k=16, inner_dim=192, dtype="bf16",
+                        zipf_s=1.5, mode=W.RoutingMode("sigmoid", False, "input"), seed=1012)
+    wl = W.make_workload_from_spec(spec)
+    _, idx, w = oracle_routing(wl)
+    ref = oracle_forward(wl, idx, 16, dtype=torch.float64).out.reshape(-1, 256)
+    emu = emulate_device_rounding(wl, idx, w).double()
+    err = (emu - ref).abs()
+    rms = float(ref.pow(2).mean().sqrt())
+    sigma = float(err.pow(2).mean().sqrt()) / rms
+    assert 5e-4 < sigma < 6e-3, sigma  # ~ 2^-9 .. 3 * 2^-9
+    assert sigma < 0.6 * RMS_TOL["bf16"]
+    rtol, atol_rel = TOL["bf16"]
+    worst = float((err / (atol_rel * rms + rtol * ref.abs())).max())
+    assert worst < 0.6, worst
+    # with atol = 2e-2 * rms the same elements come close to the bound: no room for the tail
+    assert float((err / (2e-2 * rms + rtol * ref.abs())).max()) > 0.6
