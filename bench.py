@@ -278,8 +278,11 @@ def main() -> int:
         stages[name] = ent
 
     exp_ms = stage_ms["experts"]
-    if spec.weight_dtype == "fp8":
+    if spec.weight_dtype == "fp8" and experts_hbm_bound:
         kernel = "glu_gemm_fp8w_kernel<gate,up> + <down> (fs2moe_grouped_swiglu)"
+    elif spec.weight_dtype == "fp8":
+        # e4m3 weights turned into bf16 on the way to LDS: the matrix pipe runs in bf16
+        kernel = "glu_gemm_bf16_dma_kernel<gate,up> + <down>, e4m3 weights (fs2moe_grouped_swiglu)"
     else:
         kernel = "glu_gemm_%s_dma_kernel<gate,up> + <down> (fs2moe_grouped_swiglu)" % spec.dtype
     if spec.dtype == "fp32":

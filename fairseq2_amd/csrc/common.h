@@ -138,6 +138,20 @@ __device__ __forceinline__ bf16x8 lds_read_frag_tr(const uint16_t* p_lo, const u
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// 8 e4m3 codes (two dwords) -> 8 bf16 values.
+__device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(uint32_t lo, uint32_t hi) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  u32x4 out;
+  const uint32_t w[2] = {lo, hi};
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], false);  // bytes 0, 1
+    const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], true);   // bytes 2, 3
+    out[2 * i] = (__float_as_uint(a[0]) >> 16) | (__float_as_uint(a[1]) & 0xffff0000u);
+    out[2 * i + 1] = (__float_as_uint(b[0]) >> 16) | (__float_as_uint(b[1]) & 0xffff0000u);
+  }
+  return __builtin_bit_cast(bf16x8, out);
+}
 
 // ---- host side -----------------------------------------------------------------------------------
 void set_error(const char* fmt, ...);

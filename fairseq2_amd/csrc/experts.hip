@@ -317,8 +317,73 @@ static int cu_count_by_xcd() {
   return cached;
 }
 
+// e4m3 weights go to the throughput kernel from this many rows per expert on (mean over all experts)
+#ifndef FS2MOE_FP8_GEMM_MIN_ROWS
+#define FS2MOE_FP8_GEMM_MIN_ROWS 32
+#endif
+constexpr int64_t kFp8GemmMinRowsPerExpert = FS2MOE_FP8_GEMM_MIN_ROWS;
+
 static bool dma_path_applies(int act_dtype, int D, int F) {
   return act_dtype == FS2MOE_BF16 && D % (2 * dma::BK) == 0 && F % (2 * dma::BK) == 0;
+}
+
+// The bf16 throughput kernel pair (gate/up, then down) on persistent blocks; BLAYOUT as the kernel
+// takes it, scales only with dma::W_FP8_TILED.  The caller has checked that the path applies.
+template <int BLAYOUT>
+static int launch_dma_pair(const void* x, const int32_t* row_map, const Groups& g,
+                           int64_t rows_bound, const void* w_gate, const void* w_up,
+                           const void* w_down, const float* s_gate, const float* s_up,
+                           const float* s_down, int D, int F, void* h, void* y,
+                           hipStream_t stream) {
+  using namespace dma;
+  const int groups = g.counts ? g.E : 0;
+  auto k1 = glu_gemm_bf16_dma_kernel<true, BLAYOUT>;
+  auto k2 = glu_gemm_bf16_dma_kernel<false, BLAYOUT>;
+  static bool attr_set = false;  // benign race: setting the attribute is idempotent
+  if (!attr_set) {
+    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(k1),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(k2),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+    if (e1 != hipSuccess || e2 != hipSuccess) {
+      set_error("experts: cannot reserve %d bytes of LDS: %s", SMEM_BYTES,
+                hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+      return FS2MOE_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  // Persistent blocks: one per CU (the 128 KB ring allows no more), a multiple of the 8 XCDs.
+  const int num_blocks = cu_count_by_xcd();
+  if (num_blocks == 0) {
+    set_error("experts: cannot query the compute-unit count");
+    return FS2MOE_ERR_LAUNCH;
+  }
+  const int nt1 = (F + 127) / 128, nt2 = (D + 255) / 256;
+  {
+    const int64_t m_tiles = rows_bound / BM + groups + 1;
+    if (m_tiles * nt1 > 0x7fffffffll || m_tiles * nt2 > 0x7fffffffll) {
+      set_error("experts: too many tiles");
+      return FS2MOE_ERR_UNSUPPORTED;
+    }
+  }
+  const unsigned g1 = (unsigned)num_blocks, g2 = (unsigned)num_blocks;
+  hipLaunchKernelGGL(k1, dim3(g1), dim3(NWAVES * 64), SMEM_BYTES, stream,
+                     static_cast<const uint16_t*>(x), row_map, D,
+                     static_cast<const uint16_t*>(w_gate), static_cast<const uint16_t*>(w_up), s_gate,
+                     s_up, static_cast<uint16_t*>(h), F, D, F, g, nt1);
+  if (int rc = check_launch("glu_gemm_bf16_dma<gate,up>")) return rc;
+  hipLaunchKernelGGL(k2, dim3(g2), dim3(NWAVES * 64), SMEM_BYTES, stream,
+                     static_cast<const uint16_t*>(h), static_cast<const int32_t*>(nullptr), F,
+                     static_cast<const uint16_t*>(w_down), static_cast<const uint16_t*>(nullptr),
+                     s_down, static_cast<const float*>(nullptr), static_cast<uint16_t*>(y), D, F, D, g,
+                     nt2);
+  return check_launch("glu_gemm_bf16_dma<down>");
+}
+
+// The throughput kernel addresses activations and one expert's weights with 32-bit byte offsets.
+static bool dma_offsets_fit(int64_t rows_bound, int D, int F) {
+  const int64_t wide = D > F ? D : F;
+  return rows_bound * wide * 2 <= 0xffffffffll && (int64_t)D * F * 2 <= 0xffffffffll;
 }
 
 template <int BLAYOUT>
@@ -326,52 +391,9 @@ static int launch_glu(const void* x, const int32_t* row_map, const Groups& g, in
                       const void* w_gate, const void* w_up, const void* w_down, int D, int F,
                       int act_dtype, void* h, void* y, hipStream_t stream) {
   const int groups = g.counts ? g.E : 0;
-  // The throughput kernel addresses activations and one expert's weights with 32-bit byte offsets.
-  const int64_t wide = D > F ? D : F;
-  const bool fits32 = rows_bound * wide * 2 <= 0xffffffffll && (int64_t)D * F * 2 <= 0xffffffffll;
-  if (dma_path_applies(act_dtype, D, F) && fits32) {
-    using namespace dma;
-    auto k1 = glu_gemm_bf16_dma_kernel<true, BLAYOUT>;
-    auto k2 = glu_gemm_bf16_dma_kernel<false, BLAYOUT>;
-    static bool attr_set = false;  // benign race: setting the attribute is idempotent
-    if (!attr_set) {
-      hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(k1),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
-      hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(k2),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
-      if (e1 != hipSuccess || e2 != hipSuccess) {
-        set_error("experts: cannot reserve %d bytes of LDS: %s", SMEM_BYTES,
-                  hipGetErrorString(e1 != hipSuccess ? e1 : e2));
-        return FS2MOE_ERR_LAUNCH;
-      }
-      attr_set = true;
-    }
-    // Persistent blocks: one per CU (the 128 KB ring allows no more), a multiple of the 8 XCDs.
-    const int num_blocks = cu_count_by_xcd();
-    if (num_blocks == 0) {
-      set_error("experts: cannot query the compute-unit count");
-      return FS2MOE_ERR_LAUNCH;
-    }
-    const int nt1 = (F + 127) / 128, nt2 = (D + 255) / 256;
-    {
-      const int64_t m_tiles = rows_bound / BM + groups + 1;
-      if (m_tiles * nt1 > 0x7fffffffll || m_tiles * nt2 > 0x7fffffffll) {
-        set_error("experts: too many tiles");
-        return FS2MOE_ERR_UNSUPPORTED;
-      }
-    }
-    const unsigned g1 = (unsigned)num_blocks, g2 = (unsigned)num_blocks;
-    hipLaunchKernelGGL(k1, dim3(g1), dim3(NWAVES * 64), SMEM_BYTES, stream,
-                       static_cast<const uint16_t*>(x), row_map, D,
-                       static_cast<const uint16_t*>(w_gate), static_cast<const uint16_t*>(w_up),
-                       static_cast<uint16_t*>(h), F, D, F, g, nt1);
-    if (int rc = check_launch("glu_gemm_bf16_dma<gate,up>")) return rc;
-    hipLaunchKernelGGL(k2, dim3(g2), dim3(NWAVES * 64), SMEM_BYTES, stream,
-                       static_cast<const uint16_t*>(h), static_cast<const int32_t*>(nullptr), F,
-                       static_cast<const uint16_t*>(w_down), static_cast<const uint16_t*>(nullptr),
-                       static_cast<uint16_t*>(y), D, F, D, g, nt2);
-    return check_launch("glu_gemm_bf16_dma<down>");
-  }
+  if (dma_path_applies(act_dtype, D, F) && dma_offsets_fit(rows_bound, D, F))
+    return launch_dma_pair<BLAYOUT>(x, row_map, g, rows_bound, w_gate, w_up, w_down, nullptr, nullptr,
+                                    nullptr, D, F, h, y, stream);
   if (row_map != nullptr) {
     set_error("experts: the fused gather needs bf16, D and F multiples of 64 and activation "
               "matrices below 4 GB");
@@ -455,6 +477,16 @@ extern "C" int fs2moe_grouped_swiglu(const void* xe, const int32_t* row_map, con
                 "grouped_swiglu: scales must be 16-byte aligned");
     if (max_rows == 0) return FS2MOE_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // Two regimes.  With many rows per expert the layer is a GEMM: the bf16 throughput kernel, its
+    // producers turning the codes into bf16 on the way to LDS (half the weight bytes of bf16, the
+    // same matrix rate).  With few (decode) it is a stream over the weights: the kernels below.  The
+    // row counts live on the device, so the choice goes by the mean number of rows per expert the
+    // buffers are sized for.
+    if (max_rows / E >= kFp8GemmMinRowsPerExpert && dma_offsets_fit(max_rows, D, F)) {
+      Groups g{counts, offsets, E, 0};
+      return launch_dma_pair<dma::W_FP8_TILED>(xe, row_map, g, max_rows, w_gate, w_up, w_down, s_gate,
+                                               s_up, s_down, D, F, h, ye, st);
+    }
     // Persistent blocks, three or four per CU (what the kernels' registers allow), walking work
     // items.
     // A long K is split over the 4 waves of a block (the chain of dependent loads per wave sets the

@@ -58,10 +58,21 @@ constexpr int A_BYTES = BM * 2 * BK * 2;  // 32 KB: 256 rows x 64 k
 constexpr int B_BYTES = BK * BNV * 2;     // 16 KB: one weight sub-stage of 32 k
 constexpr int UNIT_BYTES = A_BYTES + 2 * B_BYTES;  // 64 KB
 constexpr int RING_BYTES = 2 * UNIT_BYTES;         // 128 KB
+#ifndef FS2MOE_GEMM_BAND
+#define FS2MOE_GEMM_BAND 8
+#endif
+constexpr int BAND = FS2MOE_GEMM_BAND;  // row blocks per band of the tile order (see locate)
 constexpr int LIGHT_ROWS = 128;  // a last tile of at most this many rows costs about half a tile
 // after the ring: heavy-tile prefix [257], light-tile prefix [257], counts [256], offsets [256]
 constexpr int TABLE_INTS = 4 * FS2MOE_MAX_EXPERTS + 8;
-constexpr int SMEM_BYTES = RING_BYTES + TABLE_INTS * 4;
+// then, for e4m3 weights, the per-channel scales of two tiles (the one being multiplied and the one
+// whose loads are under way): [2][256] f32
+constexpr int SCALE_BYTES = 2 * BNV * 4;
+constexpr int SMEM_BYTES = RING_BYTES + TABLE_INTS * 4 + SCALE_BYTES;
+// A third weight layout next to FS2MOE_W_IN_OUT / FS2MOE_W_OUT_IN: e4m3 codes in 1 KB tiles of 16
+// output channels x 64 in-features, [expert][channel / 16][feature / 64][16][64], with one f32 scale
+// per output channel (the layout of the decode kernel in experts_fp8.h).
+constexpr int W_FP8_TILED = 2;
 }  // namespace dma
 
 // The order in which a block walks its tiles: its light tiles spread evenly among its heavy ones,
@@ -92,13 +103,19 @@ struct TileOrder {
 // BLAYOUT: FS2MOE_W_IN_OUT -- weights (Kdim, N) with N contiguous (the grouped experts), or
 // FS2MOE_W_OUT_IN -- weights (N, Kdim) with Kdim contiguous (nn.Linear: the shared expert).  In the
 // second case a unit's weights are, like its activations, 256 rows (channels) of 128 bytes: same
-// pieces, same swizzle, same plain 16-byte fragment reads.
+// pieces, same swizzle, same plain 16-byte fragment reads.  dma::W_FP8_TILED -- e4m3 codes (B0, B1
+// point at bytes) with scales S0, S1 [E, N]: a unit's weights are 16 tiles of 1 KB, half the bytes
+// of bf16; the producers turn the codes into bf16 in registers (exact) on the way to LDS and lay
+// them out as in the second case, so the consumers' main loop is the same, and the scales multiply
+// the f32 accumulators in the epilogue.
 template <bool DUAL, int BLAYOUT>
 __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     const uint16_t* __restrict__ A, const int32_t* __restrict__ row_map, int lda,
-    const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1, uint16_t* __restrict__ C,
-    int ldc, int Kdim, int N, Groups g, int n_tiles) {
+    const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
+    const float* __restrict__ S0, const float* __restrict__ S1, uint16_t* __restrict__ C, int ldc,
+    int Kdim, int N, Groups g, int n_tiles) {
   using namespace dma;
+  constexpr bool FP8 = BLAYOUT == W_FP8_TILED;
   constexpr int BN = DUAL ? 128 : 256;    // real channels per tile
   constexpr int BROW = DUAL ? 256 : 512;  // bytes per LDS row of a weight sub-tile (in x out)
   constexpr bool KN = BLAYOUT == FS2MOE_W_IN_OUT;
@@ -107,6 +124,7 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
   int32_t* s_lstart = s_hstart + FS2MOE_MAX_EXPERTS + 4;                  // [E + 1]
   int32_t* s_counts = s_lstart + FS2MOE_MAX_EXPERTS + 4;
   int32_t* s_offsets = s_counts + FS2MOE_MAX_EXPERTS;
+  float* s_scale = reinterpret_cast<float*>(smem_raw + RING_BYTES + TABLE_INTS * 4);  // [2][BNV]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -184,11 +202,10 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
   };
   auto locate = [&](int j) {
     const int logical = slot + j * grid;
-    int mt = logical / n_tiles;
-    const int nt = logical - mt * n_tiles;
-    const bool is_light = mt >= total_heavy;
+    const bool is_light = logical >= heavy_end;
+    const int in_kind = is_light ? logical - heavy_end : logical;
+    int mt = in_kind / n_tiles;  // m-tile in list order: which expert
     const int32_t* start = is_light ? s_lstart : s_hstart;
-    if (is_light) mt -= total_heavy;
     int found = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane;
@@ -198,12 +215,31 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     }
     found = __builtin_amdgcn_readfirstlane(found);
     const int off = s_offsets[found], cnt = s_counts[found];
-    const int first_row = is_light ? cnt / BM * BM : (mt - s_hstart[found]) * BM;
+    int nt, first_row;
+    if (is_light) {
+      nt = in_kind - mt * n_tiles;
+      first_row = cnt / BM * BM;
+    } else {
+      // Inside an expert the heavy tiles are numbered in bands of BAND row blocks, row block minor
+      // within a band: the 32 neighbouring tiles an XCD works on at a time then cover BAND row blocks
+      // x 32 / BAND channel blocks and find both operands in its L2 (8 + 4 slabs for 32 tiles).
+      // Channel block minor, an XCD would hold one row block x 32 channel blocks, whose weight slabs
+      // nobody else on the XCD reads: with wide layers every tile then streams its weights from
+      // memory and the kernel is bound by that.
+      const int h0 = s_hstart[found];
+      const int l = logical - h0 * n_tiles;
+      const int per_band = BAND * n_tiles;
+      const int b = l / per_band, t = l - b * per_band;
+      const int left = s_hstart[found + 1] - h0 - b * BAND;
+      const int gm = left < BAND ? left : BAND;
+      nt = t / gm;
+      first_row = (b * BAND + t - nt * gm) * BM;
+    }
     Tile t;
     t.e = found;
     t.row0 = __builtin_amdgcn_readfirstlane(off + first_row);
     t.row_end = __builtin_amdgcn_readfirstlane(off + cnt);
-    t.n0 = nt * BN;
+    t.n0 = __builtin_amdgcn_readfirstlane(nt) * BN;
     return t;
   };
 
@@ -219,14 +255,33 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     // (pieces 8..15).  The registers are the third stage of the pipeline: unit u+2 is on its way from
     // memory while unit u+1 sits in LDS and unit u is being multiplied.
     const int q = wave - CONSUMERS;
-    uint32_t pa[8], pb[KN ? 4 : 8];
+    uint32_t pa[8], pb[(KN || FP8) ? 4 : 8];
     int a_pieces = 0;  // how many of this producer's 8 activation pieces hold rows of the tile
     const uint16_t* ld_bg = B0;
     const uint16_t* ld_bu = B0;
+    // e4m3 weights: the scale of virtual channel 64 q + lane of the tile set up last, and which of
+    // the two LDS slots it goes to (tiles alternate)
+    float ld_scale = 0.f;
+    int ld_tiles = 0;
     auto setup_loads = [&](int j) {
       const Tile t = locate(j);
-      ld_bg = B0 + (size_t)t.e * wstride;
-      ld_bu = DUAL ? B1 + (size_t)t.e * wstride : ld_bg;
+      if constexpr (FP8) {
+        // wstride counts codes = bytes here; the pointers stay typed as 16-bit
+        ld_bg = reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(B0) +
+                                                  (size_t)t.e * wstride);
+        ld_bu = DUAL ? reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(B1) +
+                                                         (size_t)t.e * wstride)
+                     : ld_bg;
+        const int v = 64 * q + lane;  // virtual channel of the tile: gate 0..127, up 128..255
+        const bool up = DUAL && v >= 128;
+        int ch = t.n0 + (up ? v - 128 : v);
+        ch = ch < N ? ch : N - 1;  // clamped channels are never stored
+        ld_scale = (up ? S1 : S0)[(size_t)t.e * N + ch];
+        ++ld_tiles;
+      } else {
+        ld_bg = B0 + (size_t)t.e * wstride;
+        ld_bu = DUAL ? B1 + (size_t)t.e * wstride : ld_bg;
+      }
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
         const int p = q + 4 * jj;
@@ -244,7 +299,18 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
       const int rows = t.row_end - t.row0;
       a_pieces = rows >= BM ? 8 : (rows - 8 * q + 31) / 32;
       a_pieces = a_pieces < 0 ? 0 : a_pieces;
-      if constexpr (KN) {
+      if constexpr (FP8) {
+        // a unit's weights are the 16 tiles (channel group gi = q + 4 jj of the 256 virtual channels,
+        // k block ku); with DUAL groups 0..7 are gate channels and 8..15 the same up channels
+        const int nkb = Kdim / (2 * BK);
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const int gi = q + 4 * jj;
+          int group = t.n0 / 16 + (DUAL ? (gi & 7) : gi);
+          group = group < N / 16 ? group : N / 16 - 1;  // clamped channels are never stored
+          pb[jj] = (uint32_t)(((size_t)group * nkb) * 1024 + lane * 16);
+        }
+      } else if constexpr (KN) {
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
           // piece r of a sub-tile = 1024 / BROW consecutive k rows
@@ -270,15 +336,25 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
         }
       }
     };
-    u32x4 stage[16];
+    u32x4 stage[FP8 ? 12 : 16];
     int stage_pieces = 0;  // a_pieces of the unit held in `stage`
+    int stage_scale_slot = -1;  // e4m3: the unit in `stage` is the first of a tile with this slot
+    float stage_scale = 0.f;
     // Unit ku of the tile set up last -> registers.
     auto load_unit = [&](int ku) {
       const uint8_t* abase = reinterpret_cast<const uint8_t*>(A + (size_t)ku * (2 * BK));
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj)
         if (jj < a_pieces) stage[jj] = *reinterpret_cast<const u32x4*>(abase + pa[jj]);
-      if constexpr (KN) {
+      if constexpr (FP8) {
+        const uint8_t* bg = reinterpret_cast<const uint8_t*>(ld_bg) + (size_t)ku * 1024;
+        const uint8_t* bu = reinterpret_cast<const uint8_t*>(ld_bu) + (size_t)ku * 1024;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+          stage[8 + jj] = *reinterpret_cast<const u32x4*>((jj < 2 ? bg : bu) + pb[jj]);
+        stage_scale_slot = ku == 0 ? ((ld_tiles - 1) & 1) : -1;
+        stage_scale = ld_scale;
+      } else if constexpr (KN) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           const size_t k0 = ((size_t)ku * 2 + h) * BK * N;
@@ -306,11 +382,29 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj)
         if (jj < stage_pieces) *reinterpret_cast<u32x4*>(dst + jj * 4096) = stage[jj];
-      // weights: in x out -- sub-stage h, pieces q + 4 j; out x in -- pieces q + 4 jj of the 32 KB
-      // block.  Either way stage[8 + i] goes to byte offset i * 4096 of the weight area.
+      if constexpr (FP8) {
+        // Tile gi = q + 4 jj holds channel rows 16 gi .. 16 gi + 15 of the weight block; the lane's 16
+        // codes are k 16 (lane % 4) .. +15 of row 16 gi + lane / 4, i.e. chunks 2 (lane % 4) and the
+        // next one of that 128-byte row, stored where the fragment reads expect them (chunk kc of
+        // row r in slot kc ^ ((r >> 1) & 7); 16 gi does not change the key).
+        const int r = lane >> 2, kc = 2 * (lane & 3), key = (lane >> 3) & 7;
+        uint8_t* wdst = smem_raw + half * UNIT_BYTES + A_BYTES + (16 * q + r) * 128;
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        *reinterpret_cast<u32x4*>(dst + A_BYTES + i * 4096) = stage[8 + i];
+        for (int jj = 0; jj < 4; ++jj) {
+          const u32x4 c = stage[8 + jj];
+          *reinterpret_cast<bf16x8*>(wdst + jj * 8192 + ((kc ^ key) << 4)) =
+              fp8x8_to_bf16x8(c[0], c[1]);
+          *reinterpret_cast<bf16x8*>(wdst + jj * 8192 + (((kc + 1) ^ key) << 4)) =
+              fp8x8_to_bf16x8(c[2], c[3]);
+        }
+        if (stage_scale_slot >= 0) s_scale[stage_scale_slot * BNV + 64 * q + lane] = stage_scale;
+      } else {
+        // weights: in x out -- sub-stage h, pieces q + 4 j; out x in -- pieces q + 4 jj of the 32 KB
+        // block.  Either way stage[8 + i] goes to byte offset i * 4096 of the weight area.
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          *reinterpret_cast<u32x4*>(dst + A_BYTES + i * 4096) = stage[8 + i];
+      }
     };
     TileOrder order(my_heavy, my_tiles - my_heavy, (int)(blockIdx.x & 7));
     int ld_ku = -1;  // unit (within its tile) loaded last
@@ -413,7 +507,7 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
   // Chunk c of row r sits at r * ROWB + ((c ^ key(r)) << 4), key(r) = (r >> 1) & 7 when DUAL (rows are
   // 128 B: two rows span the banks) and r & 15 otherwise.  With r and c split into a per-lane part and
   // a compile-time part, every address below is one per-lane base XOR / plus constants.
-  auto store_tile = [&](const Tile& t, int gu) {
+  auto store_tile = [&](const Tile& t, int gu, int scale_slot) {
     constexpr int ROWB = DUAL ? 128 : 256;  // bytes per row of the wave's output tile
     constexpr int CH = ROWB / 16;           // 16-byte chunks per row
     constexpr int RPI = 64 / CH;            // rows per store instruction
@@ -443,12 +537,29 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           float v[4];
+          if constexpr (FP8) {
+            // the lane's four channels 8 q + 4 lk + {0..3} of fragment fn: virtual channel c of the
+            // tile (and 128 + c for the up half)
+            const int c = (DUAL ? wn * 64 : wn * 128) + fn * 32 + 8 * q + 4 * lk;
+            const float* sc = s_scale + scale_slot * BNV + c;
+            const f32x4 sg = *reinterpret_cast<const f32x4*>(sc);
+            if constexpr (DUAL) {
+              const f32x4 su = *reinterpret_cast<const f32x4*>(sc + 128);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            if (DUAL)
-              v[j] = silu_f32(acc[fn][fm][4 * q + j]) * acc[fn + 2][fm][4 * q + j];
-            else
-              v[j] = acc[fn][fm][4 * q + j];
+              for (int j = 0; j < 4; ++j)
+                v[j] = silu_f32(acc[fn][fm][4 * q + j] * sg[j]) * (acc[fn + 2][fm][4 * q + j] * su[j]);
+            } else {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) v[j] = acc[fn][fm][4 * q + j] * sg[j];
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              if (DUAL)
+                v[j] = silu_f32(acc[fn][fm][4 * q + j]) * acc[fn + 2][fm][4 * q + j];
+              else
+                v[j] = acc[fn][fm][4 * q + j];
+            }
           }
           u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
           *reinterpret_cast<u32x2*>(buf + (wbase_l ^ (uint32_t)((4 * fn + q) << 4))) = o;
@@ -472,7 +583,7 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
   TileOrder order(my_heavy, my_tiles - my_heavy, (int)(blockIdx.x & 7));
   Tile cur = locate(order.next());
   bool wave_active = cur.row0 + wm * 64 < cur.row_end;
-  int ku = 0, tiles_left = my_tiles - 1;
+  int ku = 0, tiles_left = my_tiles - 1, tiles_done = 0;
   for (int gu = 0; gu < total_units; ++gu) {
     __syncthreads();  // the producers have seen unit gu land
     if (ku == 0) {
@@ -486,7 +597,8 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     if (wave_active) compute_unit(gu);
     if (++ku == nu) {
       __syncthreads();  // every consumer is done with the ring half the epilogue borrows
-      if (wave_active) store_tile(cur, gu);
+      if (wave_active) store_tile(cur, gu, tiles_done & 1);
+      ++tiles_done;
       ku = 0;
       if (tiles_left-- > 0) {
         cur = locate(order.next());

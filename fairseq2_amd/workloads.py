@@ -1,8 +1,9 @@
 """Seeded synthetic workloads for the MoE feed-forward path.
 
-Five named layer shapes are defined: one small fp32 case that the CPU reference
+Six named layer shapes are defined: one small fp32 case that the CPU reference
 formulation runs comfortably, three bf16 prefill shapes (Mixtral-8x7B,
-Qwen3-30B-A3B, Llama-4-Scout) and one fp8-weight decode shape.  Every tensor is
+Qwen3-30B-A3B, Llama-4-Scout), the Qwen3 prefill shape with fp8 weights and one
+fp8-weight decode shape.  Every tensor is
 drawn from one CPU generator in a fixed order, so the same seed gives the same
 layer on any machine:
 
@@ -95,6 +96,11 @@ SPECS: dict[str, WorkloadSpec] = {
     ),
     "llama4_scout": WorkloadSpec(
         "llama4_scout", 3, 8, 1024, 5120, 16, 1, 8192, "bf16", "bf16", None, True, _REFERENCE_MODE
+    ),
+    # the Qwen3 prefill shape with the decode case's weight format: e4m3 weights in the GEMM regime
+    "qwen3_30b_a3b_fp8": WorkloadSpec(
+        "qwen3_30b_a3b_fp8", 2, 8, 1024, 2048, 128, 8, 768, "bf16", "fp8", 1.2, False,
+        RoutingMode("softmax", True, "output"),
     ),
     "qwen3_decode_fp8": WorkloadSpec(
         "qwen3_decode_fp8", 4, 64, 1, 2048, 128, 8, 768, "bf16", "fp8", 1.2, False,

@@ -190,6 +190,16 @@ def test_llama4_scout_shape(gpu_device):
     _full_size_case("llama4_scout", gpu_device, sample=256)
 
 
+def test_qwen3_prefill_shape_with_fp8_weights(gpu_device):
+    # 512 rows per expert on average: e4m3 weights go through the throughput kernel.  Same seed as the
+    # bf16 case, so the routing is the same; the reference is evaluated on the de-quantised weights.
+    wl, m, x, out, disp = _full_size_case("qwen3_30b_a3b_fp8", gpu_device, sample=256)
+    assert m.experts.has_fp8_weights
+    assert sorted(disp.counts.cpu().tolist(), reverse=True)[:5] == [8138, 7691, 6939, 6074, 5198]
+    with torch.no_grad():
+        assert torch.equal(m(x), out), "deterministic"
+
+
 def test_qwen3_decode_fp8_shape(gpu_device):
     # Decode regime with e4m3 weights and per-output-channel scales.  The reference of the comparison
     # is the f32 evaluation with the de-quantised weights, so the bound is the bf16 one; the

@@ -331,10 +331,10 @@ def test_grouped_swiglu_beyond_4_gb_of_activations(gpu_device):
         _abi.grouped_swiglu(xe, counts.to(dev), offsets.to(dev), wg.to(dev), wu.to(dev), wd.to(dev), e, row_map=row_map)
 
 
-def test_grouped_swiglu_fp8_row_map_equals_gathered_rows(gpu_device):
+@pytest.mark.parametrize("t,d,e,k,f", [(48, 128, 16, 4, 64), (700, 128, 4, 2, 192)])  # decode / throughput kernel
+def test_grouped_swiglu_fp8_row_map_equals_gathered_rows(gpu_device, t, d, e, k, f):
     """The e4m3-weight kernels read rows through the permutation too, with identical results."""
-    _say("grouped_swiglu fp8 row_map")
-    t, d, e, k, f = 48, 128, 16, 4, 64
+    _say("grouped_swiglu fp8 row_map", t, d, e, k, f)
     spec = W.small_spec(tokens=t, model_dim=d, num_experts=e, top_k=k, inner_dim=f, dtype="bf16",
                         weight_dtype="fp8", zipf_s=1.2, seed=17)
     wl = W.make_workload_from_spec(spec)
@@ -417,6 +417,12 @@ def test_combine_matches_oracle(gpu_device, dtype, weight_output, with_base, k):
     [
         ([5, 0, 17, 64, 1, 11, 0, 33], 128, 192),  # decode-like: few rows, empty experts
         ([100, 3], 64, 64),  # more than 64 rows: weights re-streamed per 64-row chunk
+        # 64 or more rows per expert on average: the throughput kernel (codes turned into bf16 on
+        # the way to LDS, scales in its epilogue); ragged last tiles, an empty expert, F and D that
+        # leave the last channel tile partly (192 = 128 + 64) or mostly (128 of 256) empty
+        ([300, 0, 70, 513, 1, 129, 256, 40], 128, 192),
+        ([700, 260], 64, 64),
+        ([257, 255, 31, 1000], 320, 448),
     ],
 )
 def test_grouped_swiglu_fp8_weights_match_oracle(gpu_device, rows_per_expert, d, f):
