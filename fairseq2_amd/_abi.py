@@ -15,10 +15,11 @@ from torch import Tensor
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfs2moe.so")
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
+W_IN_OUT, W_OUT_IN = 0, 1
 MAX_EXPERTS, MAX_TOP_K = 256, 16
 
 # name -> (restype, argtypes); mirrors include/fs2moe.h one to one
@@ -83,6 +84,31 @@ _PROTOTYPES = {
     "fs2moe_forward_static": (
         c_int32,
         [c_void_p] * 13 + [c_int32] * 12 + [c_void_p, c_void_p],
+    ),
+    "fs2moe_grouped_gemm": (
+        c_int32,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32,
+         c_int64, c_int32, c_void_p, c_void_p],
+    ),
+    "fs2moe_grouped_wgrad": (
+        c_int32,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int64,
+         c_int32, c_void_p, c_void_p],
+    ),
+    "fs2moe_swiglu_backward": (
+        c_int32,
+        [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
+         c_void_p],
+    ),
+    "fs2moe_pair_dot": (
+        c_int32,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p,
+         c_void_p],
+    ),
+    "fs2moe_router_backward": (
+        c_int32,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32,
+         c_int32, c_void_p, c_void_p],
     ),
     "fs2moe_forward_norm": (
         c_int32,
@@ -428,6 +454,152 @@ def combine(
         )
         _check(rc, "fs2moe_combine_residual")
     return out
+
+
+# ---------------------------------------------------------------------------------- backward pass
+def _same(name: str, t: Tensor, shape: tuple, dtype: torch.dtype, dev: torch.device) -> None:
+    if tuple(t.shape) != tuple(shape) or t.dtype != dtype or t.device != dev or not t.is_contiguous():
+        raise ValueError(
+            f"{name} must be a contiguous {tuple(shape)} {dtype} tensor on {dev}, got {tuple(t.shape)} "
+            f"{t.dtype} on {t.device}")
+
+
+def grouped_gemm(
+    a: Tensor,
+    b: Tensor,
+    layout: int,
+    counts: Tensor | None = None,
+    offsets: Tensor | None = None,
+    num_experts: int = 1,
+    row_map: Tensor | None = None,
+    rows: int | None = None,
+) -> Tensor:
+    """``c[r] = a[r] @ B_e`` for the rows ``r`` of every expert ``e`` (``fs2moe_grouped_gemm``).
+
+    ``b`` holds one ``(K, N)`` matrix per expert, ``layout`` ``W_IN_OUT``: ``(E*K, N)``, or
+    ``W_OUT_IN``: ``(E*N, K)`` -- i.e. the second form multiplies by the transpose of what the
+    forward pass multiplied by in the first.  Without ``counts`` all rows belong to one matrix.  With
+    ``row_map``, row ``r`` of the product is computed from ``a[row_map[r]]`` and ``rows`` is the
+    number of rows of the result."""
+    lib = load()
+    e = num_experts
+    k = a.shape[1]
+    if b.dim() != 2 or b.dtype != a.dtype or b.device != a.device or not b.is_contiguous() or b.numel() % (e * k):
+        raise ValueError("b must hold one (K, N) or (N, K) matrix per expert in the dtype of a")
+    n = b.numel() // (e * k)
+    _same("b", b, (e * k, n) if layout == W_IN_OUT else (e * n, k), a.dtype, a.device)
+    if (counts is None) != (offsets is None):
+        raise ValueError("counts and offsets come together")
+    if counts is not None:
+        _same("counts", counts, (e,), torch.int32, a.device)
+        _same("offsets", offsets, (e + 1,), torch.int32, a.device)
+    elif e != 1:
+        raise ValueError("a dense product has one matrix")
+    if row_map is not None:
+        if rows is None:
+            rows = row_map.shape[0]
+        _same("row_map", row_map, (row_map.shape[0],), torch.int32, a.device)
+        if row_map.shape[0] < rows:
+            raise ValueError("row_map is shorter than the result")
+    else:
+        rows = a.shape[0]
+    c = torch.empty((rows, n), dtype=a.dtype, device=a.device)
+    rc = lib.fs2moe_grouped_gemm(
+        _ptr(a), _ptr(row_map), _ptr(counts), _ptr(offsets), _ptr(b), layout, e, k, n, rows,
+        dtype_code(a.dtype), _ptr(c), _stream(),
+    )
+    _check(rc, "fs2moe_grouped_gemm")
+    return c
+
+
+def grouped_wgrad(
+    a: Tensor,
+    b: Tensor,
+    counts: Tensor | None = None,
+    offsets: Tensor | None = None,
+    num_experts: int = 1,
+    a_row_map: Tensor | None = None,
+) -> Tensor:
+    """``dw_e = A_e^T @ B_e`` over the rows of each expert: ``(E*M, N)`` (``fs2moe_grouped_wgrad``).
+    ``b`` has one row per row of the experts' buffer; ``a`` as well, or, with ``a_row_map``, row
+    ``r`` of ``A`` is ``a[a_row_map[r]]``."""
+    lib = load()
+    e = num_experts
+    rows, n = b.shape
+    m = a.shape[1]
+    if a.dtype != b.dtype or a.device != b.device or not a.is_contiguous() or not b.is_contiguous():
+        raise ValueError("a and b must be contiguous tensors of one dtype on one device")
+    if (counts is None) != (offsets is None):
+        raise ValueError("counts and offsets come together")
+    if counts is not None:
+        _same("counts", counts, (e,), torch.int32, a.device)
+        _same("offsets", offsets, (e + 1,), torch.int32, a.device)
+    elif e != 1:
+        raise ValueError("a dense product has one matrix")
+    if a_row_map is not None:
+        _same("a_row_map", a_row_map, (a_row_map.shape[0],), torch.int32, a.device)
+        if a_row_map.shape[0] < rows:
+            raise ValueError("a_row_map is shorter than b")
+    elif a.shape[0] != rows:
+        raise ValueError("a and b must have the same number of rows")
+    dw = torch.empty((e * m, n), dtype=a.dtype, device=a.device)
+    rc = lib.fs2moe_grouped_wgrad(
+        _ptr(a), _ptr(a_row_map), _ptr(b), _ptr(counts), _ptr(offsets), e, m, n, rows,
+        dtype_code(a.dtype), _ptr(dw), _stream(),
+    )
+    _check(rc, "fs2moe_grouped_wgrad")
+    return dw
+
+
+def swiglu_backward(g: Tensor, u: Tensor, dh: Tensor) -> tuple[Tensor, Tensor, Tensor]:
+    """``(h, dg, du)`` of ``h = SiLU(g) * u`` given ``dh``; ``dg`` and ``du`` overwrite ``g`` and ``u``."""
+    lib = load()
+    _same("u", u, g.shape, g.dtype, g.device)
+    _same("dh", dh, g.shape, g.dtype, g.device)
+    if not g.is_contiguous():
+        raise ValueError("g must be contiguous")
+    h = torch.empty_like(g)
+    rc = lib.fs2moe_swiglu_backward(
+        _ptr(g), _ptr(u), _ptr(dh), g.shape[0], g.shape[1], dtype_code(g.dtype), _ptr(h), _ptr(g),
+        _ptr(u), _stream(),
+    )
+    _check(rc, "fs2moe_swiglu_backward")
+    return h, g, u
+
+
+def pair_dot(a: Tensor, a_rows: Tensor, b: Tensor, a2: Tensor | None = None) -> Tensor:
+    """``out[t, k] = <a[a_rows[t, k]] (+ a2[a_rows[t, k]]), b[t]>`` in f32 (``fs2moe_pair_dot``)."""
+    lib = load()
+    t, k = a_rows.shape
+    d = b.shape[1]
+    _same("a_rows", a_rows, (t, k), torch.int32, b.device)
+    _same("b", b, (t, d), a.dtype, a.device)
+    _same("a", a, (a.shape[0], d), a.dtype, a.device)
+    if a2 is not None:
+        _same("a2", a2, a.shape, a.dtype, a.device)
+    out = torch.empty((t, k), dtype=torch.float32, device=b.device)
+    rc = lib.fs2moe_pair_dot(_ptr(a), _ptr(a2), _ptr(a_rows), _ptr(b), t, k, d, dtype_code(a.dtype),
+                             _ptr(out), _stream())
+    _check(rc, "fs2moe_pair_dot")
+    return out
+
+
+def router_backward(logits: Tensor, topk_idx: Tensor, topk_w: Tensor, d_w: Tensor, score_fn: int,
+                    renormalize: bool, dtype: torch.dtype) -> Tensor:
+    """Gradient of the combine weights -> gradient of the logits ``(T, E)`` in ``dtype``."""
+    lib = load()
+    t, e = logits.shape
+    k = topk_idx.shape[1]
+    dev = logits.device
+    _same("logits", logits, (t, e), torch.float32, dev)
+    _same("topk_idx", topk_idx, (t, k), torch.int32, dev)
+    _same("topk_w", topk_w, (t, k), torch.float32, dev)
+    _same("d_w", d_w, (t, k), torch.float32, dev)
+    dl = torch.empty((t, e), dtype=dtype, device=dev)
+    rc = lib.fs2moe_router_backward(_ptr(logits), _ptr(topk_idx), _ptr(topk_w), _ptr(d_w), t, e, k,
+                                    score_fn, int(renormalize), dtype_code(dtype), _ptr(dl), _stream())
+    _check(rc, "fs2moe_router_backward")
+    return dl
 
 
 def check_layer_arguments(x, router, router_bias, w_gate, w_up, w_down, num_experts, f, scales, shared) -> None:

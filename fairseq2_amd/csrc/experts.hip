@@ -545,6 +545,96 @@ extern "C" int fs2moe_grouped_swiglu(const void* xe, const int32_t* row_map, con
                                      h, ye, static_cast<hipStream_t>(stream));
 }
 
+// One grouped (or dense) GEMM, C = A @ B_e, on the kernels of the SwiGLU pair's second half.
+template <int BLAYOUT>
+static int launch_gemm(const void* a, const int32_t* row_map, const Groups& g, int64_t rows_bound,
+                       const void* b, int K, int N, int dtype, void* c, hipStream_t stream) {
+  const int groups = g.counts ? g.E : 0;
+  if (dtype == FS2MOE_BF16 && K % (2 * dma::BK) == 0 && dma_offsets_fit(rows_bound, K, N)) {
+    using namespace dma;
+    auto k = glu_gemm_bf16_dma_kernel<false, BLAYOUT>;
+    static bool attr_set = false;  // benign race: setting the attribute is idempotent
+    if (!attr_set) {
+      hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(k),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+      if (e1 != hipSuccess) {
+        set_error("gemm: cannot reserve %d bytes of LDS: %s", SMEM_BYTES, hipGetErrorString(e1));
+        return FS2MOE_ERR_LAUNCH;
+      }
+      attr_set = true;
+    }
+    const int num_blocks = cu_count_by_xcd();
+    if (num_blocks == 0) {
+      set_error("gemm: cannot query the compute-unit count");
+      return FS2MOE_ERR_LAUNCH;
+    }
+    const int nt = (N + 255) / 256;
+    if ((rows_bound / BM + groups + 1) * nt > 0x7fffffffll) {
+      set_error("gemm: too many tiles");
+      return FS2MOE_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(k, dim3((unsigned)num_blocks), dim3(NWAVES * 64), SMEM_BYTES, stream,
+                       static_cast<const uint16_t*>(a), row_map, K, static_cast<const uint16_t*>(b),
+                       static_cast<const uint16_t*>(nullptr), static_cast<const float*>(nullptr),
+                       static_cast<const float*>(nullptr), static_cast<uint16_t*>(c), N, K, N, g, nt);
+    return check_launch("glu_gemm_bf16_dma<single>");
+  }
+  if (row_map != nullptr) {
+    set_error("gemm: a row map needs bf16, K a multiple of 64 and matrices below 4 GB");
+    return FS2MOE_ERR_UNSUPPORTED;
+  }
+  if (dtype == FS2MOE_BF16) {
+    using namespace bf16k;
+    const int64_t m_tiles = rows_bound / BM + groups + 1;
+    const int nt = (N + BN - 1) / BN;
+    if (m_tiles * nt > 0x7fffffffll) {
+      set_error("gemm: grid too large");
+      return FS2MOE_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL((glu_gemm_bf16_kernel<false, BLAYOUT>), dim3((unsigned)(m_tiles * nt)),
+                       dim3(256), 0, stream, static_cast<const uint16_t*>(a), K,
+                       static_cast<const uint16_t*>(b), static_cast<const uint16_t*>(nullptr),
+                       static_cast<uint16_t*>(c), N, K, N, g, nt);
+    return check_launch("glu_gemm_bf16<single>");
+  }
+  using namespace f32k;
+  const int64_t m_tiles = rows_bound / BM + groups + 1;
+  const int nt = (N + BN - 1) / BN;
+  if (m_tiles * nt > 0x7fffffffll) {
+    set_error("gemm: grid too large");
+    return FS2MOE_ERR_UNSUPPORTED;
+  }
+  hipLaunchKernelGGL((glu_gemm_f32_kernel<false, BLAYOUT>), dim3((unsigned)(m_tiles * nt)), dim3(256),
+                     0, stream, static_cast<const float*>(a), K, static_cast<const float*>(b),
+                     static_cast<const float*>(nullptr), static_cast<float*>(c), N, K, N, g, nt);
+  return check_launch("glu_gemm_f32<single>");
+}
+
+extern "C" int fs2moe_grouped_gemm(const void* a, const int32_t* row_map, const int32_t* counts,
+                                   const int32_t* offsets, const void* b, int32_t b_layout,
+                                   int32_t E, int32_t K, int32_t N, int64_t max_rows, int32_t dtype,
+                                   void* c, void* stream) {
+  FS2_REQUIRE(a && b && c, "grouped_gemm: null pointer");
+  FS2_REQUIRE((counts == nullptr) == (offsets == nullptr), "grouped_gemm: counts without offsets");
+  FS2_REQUIRE(E >= 1 && E <= FS2MOE_MAX_EXPERTS && (counts != nullptr || E == 1),
+              "grouped_gemm: E=%d", E);
+  FS2_REQUIRE(b_layout == FS2MOE_W_IN_OUT || b_layout == FS2MOE_W_OUT_IN, "grouped_gemm: layout %d",
+              b_layout);
+  FS2_REQUIRE(dtype == FS2MOE_F32 || dtype == FS2MOE_BF16, "grouped_gemm: dtype %d", dtype);
+  FS2_REQUIRE(K > 0 && N > 0 && K % 8 == 0 && N % 8 == 0,
+              "grouped_gemm: K=%d and N=%d must be positive multiples of 8", K, N);
+  FS2_REQUIRE(max_rows >= 0 && max_rows < (1ll << 31), "grouped_gemm: max_rows=%lld",
+              (long long)max_rows);
+  FS2_REQUIRE(aligned16(a) && aligned16(b) && aligned16(c),
+              "grouped_gemm: buffers must be 16-byte aligned");
+  if (max_rows == 0) return FS2MOE_OK;
+  Groups g{counts, offsets, E, (int)max_rows};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (b_layout == FS2MOE_W_IN_OUT)
+    return launch_gemm<FS2MOE_W_IN_OUT>(a, row_map, g, max_rows, b, K, N, dtype, c, st);
+  return launch_gemm<FS2MOE_W_OUT_IN>(a, row_map, g, max_rows, b, K, N, dtype, c, st);
+}
+
 extern "C" int fs2moe_dense_swiglu(const void* x, const void* w_gate, const void* w_up,
                                    const void* w_down, int32_t T, int32_t D, int32_t F,
                                    int32_t act_dtype, void* h, void* y, void* stream) {

@@ -409,6 +409,10 @@ class MoE(FeedForwardNetwork):
         seqs = self._autocast(seqs)
         if residual is not None:
             residual = self._autocast(residual)
+        if torch.is_grad_enabled() and any(
+            t is not None and t.requires_grad for t in (seqs, residual, *self.parameters())
+        ):
+            return self._differentiable(seqs, residual, norm)
         x = self._checked_rows(seqs)
         norm_args = self._norm_args(norm, x)
         res = None
@@ -424,6 +428,53 @@ class MoE(FeedForwardNetwork):
         if type(ex) is GroupedExpertNetwork and (se is None or type(se) is GLUFeedForwardNetwork):
             return self._single_call(x, res, norm_args).view(seqs.shape)
         return self._stages(x, res, norm_args)[0].view(seqs.shape)
+
+    def _differentiable(self, seqs: Tensor, residual: Tensor | None, norm) -> Tensor:
+        """The training path: the layer as one ``torch.autograd.Function`` whose backward pass runs
+        on the library's kernels (:mod:`fairseq2_amd.autograd`), for ``seqs``, ``residual`` and
+        every parameter.  Covers the reference configuration and the routing extensions; the fused
+        normalisation, e4m3 weights and other expert modules are forward-only."""
+        ex, se = self.experts, self.shared_expert
+        why = None
+        if norm is not None:
+            why = "the normalisation fused into the router has no backward pass (normalise outside the layer)"
+        elif type(ex) is not GroupedExpertNetwork or (se is not None and type(se) is not GLUFeedForwardNetwork):
+            why = "only GroupedExpertNetwork experts and a GLUFeedForwardNetwork shared expert are differentiated"
+        elif ex.has_fp8_weights:
+            why = "e4m3 expert weights are an inference format"
+        elif ex.num_local_experts % 8:
+            why = "the router's backward kernels need a number of experts that is a multiple of 8"
+        if why is not None:
+            raise RuntimeError(
+                f"fairseq2_amd.MoE: {why}; call it under torch.no_grad() / torch.inference_mode(), "
+                "or freeze the inputs and the module with requires_grad_(False)")
+        x = self._checked_rows(seqs, allow_grad=True)
+        res = None
+        if residual is not None:
+            if residual.shape != seqs.shape or residual.dtype != seqs.dtype:
+                raise ValueError("residual must have the shape and dtype of seqs")
+            _require_device(residual)
+            res = residual.reshape(-1, seqs.shape[-1]).contiguous()
+        if x.shape[0] == 0:
+            return torch.empty_like(seqs)
+        from fairseq2_amd.autograd import MoEFunction
+
+        shared = (None, None, None)
+        if se is not None:
+            shared = (se.gate_proj.weight, se.inner_proj.weight, se.output_proj.weight)
+        _abi.check_layer_arguments(
+            x.detach(), self.router.detach(), self.router_bias, ex.gate_proj.detach(),
+            ex.inner_proj.detach(), ex.output_proj.detach(), ex.num_local_experts, ex.inner_dim, None,
+            None if se is None else tuple(t.detach() for t in shared),
+        )
+        cfg = dict(
+            num_experts=ex.num_local_experts, top_k=self.top_k, tile_m=self.tile_m,
+            score_fn=_SCORE_FNS[self.score_fn], renormalize=self.renormalize,
+            scale_input=self.scale_on == "input", router_bias=self.router_bias,
+        )
+        out = MoEFunction.apply(x, res, self.router, ex.gate_proj, ex.inner_proj, ex.output_proj,
+                                *shared, cfg)
+        return out.view(seqs.shape)
 
     def _autocast(self, t: Tensor) -> Tensor:
         if t.is_cuda and torch.is_autocast_enabled("cuda"):
@@ -526,12 +577,13 @@ class MoE(FeedForwardNetwork):
         out, idx, w, disp = self._stages(x)
         return out.view(seqs.shape), idx, w, disp
 
-    def _checked_rows(self, seqs: Tensor) -> Tensor:
+    def _checked_rows(self, seqs: Tensor, allow_grad: bool = False) -> Tensor:
         """Validates ``seqs`` against the module and returns it as contiguous ``(T, dim)`` rows."""
         if self.tp_gang is not None:
             raise NotImplementedError("tensor-parallel reduction is not part of the single-GPU path")
         _require_device(seqs)
-        _require_forward_only(seqs, *self.parameters())
+        if not allow_grad:
+            _require_forward_only(seqs, *self.parameters())
         if seqs.dtype != self.router.dtype:
             hint = ""
             if torch.is_autocast_enabled("cuda"):

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FS2MOE_ABI_VERSION 7
+#define FS2MOE_ABI_VERSION 8
 
 /* element types */
 #define FS2MOE_F32 0
@@ -261,6 +261,64 @@ int fs2moe_forward_static(const void* x, const void* residual, const void* route
                           int32_t F, int32_t F_shared, int32_t tile_m, int32_t act_dtype,
                           int32_t w_dtype, int32_t score_fn, int32_t renormalize,
                           int32_t scale_input, void* out, void* stream);
+
+/*
+ * ---- Backward pass ------------------------------------------------------------------------------
+ * The reference layer is differentiated by torch.autograd (the trainer calls backward on the loss,
+ * trainer.py:586-587); the entry points below, together with fs2moe_dispatch (the gather of output
+ * gradients into expert order) and fs2moe_combine (the scatter of input gradients back to token
+ * order), are what that derivation needs of the device.
+ *
+ * One grouped GEMM: c[r] = a[r] @ B_e for the rows r of every expert e.
+ * Replaces one torch.bmm of experts.py:107-112, or its transpose in the backward pass (the input
+ * gradient of x @ W is dy @ W^T: the same weights read in the other orientation), or one F.linear of
+ * ffn.py:374-395.
+ *   a [rows, K] dtype (through row_map as in fs2moe_grouped_swiglu, when given)
+ *   b  FS2MOE_W_IN_OUT: [E*K, N], FS2MOE_W_OUT_IN: [E*N, K]          c [max_rows, N] dtype (out)
+ *   counts/offsets NULL: one matrix (E = 1) and max_rows rows.  K and N multiples of 8.
+ */
+int fs2moe_grouped_gemm(const void* a, const int32_t* row_map, const int32_t* counts,
+                        const int32_t* offsets, const void* b, int32_t b_layout, int32_t E, int32_t K,
+                        int32_t N, int64_t max_rows, int32_t dtype, void* c, void* stream);
+
+/*
+ * Weight gradient: dw_e [M, N] = A_e^T @ B_e, the contraction running over the rows of expert e
+ * (zero for an expert without rows).  What autograd derives for the weights of experts.py:107-112
+ * (A = the experts' input rows or h, B = the gradient of the product) and of ffn.py:374-395.
+ *   a [rows, M] dtype (row r read from a[a_row_map[r]] when a_row_map is given)   b [rows, N] dtype
+ *   dw [E*M, N] dtype (out).  M and N multiples of 8 (bf16) or 4 (f32).
+ */
+int fs2moe_grouped_wgrad(const void* a, const int32_t* a_row_map, const void* b,
+                         const int32_t* counts, const int32_t* offsets, int32_t E, int32_t M,
+                         int32_t N, int64_t max_rows, int32_t dtype, void* dw, void* stream);
+
+/*
+ * SwiGLU backward, element-wise: h = SiLU(g) * u, dg = dh * u * SiLU'(g), du = dh * SiLU(g).
+ * The derivative of experts.py:110-111 / ffn.py:384-391.  h, dg, du may alias g, u, dh element for
+ * element.     all [rows, F] dtype
+ */
+int fs2moe_swiglu_backward(const void* g, const void* u, const void* dh, int64_t rows, int32_t F,
+                           int32_t dtype, void* h, void* dg, void* du, void* stream);
+
+/*
+ * Gradient of the combine weights: out[t, k] = <a[a_rows[t, k]] (+ a2[a_rows[t, k]]), b[t]> in f32.
+ * The derivative of the scaling of moe.py:132-134 (a = the gradient of the scaled rows, b = x) or,
+ * when the weights scale the experts' output, of the weighted sum (a = ye, b = the output gradient).
+ *   a, a2 [rows, D] dtype (a2 may be NULL)   a_rows [T, K] int32   b [T, D] dtype   out [T, K] f32
+ */
+int fs2moe_pair_dot(const void* a, const void* a2, const int32_t* a_rows, const void* b, int32_t T,
+                    int32_t K, int32_t D, int32_t dtype, float* out, void* stream);
+
+/*
+ * Router backward: gradient of the K combine weights -> gradient of all E logits of each token
+ * (zero where the score function does not reach).  The derivative of moe.py:113-127 with the score
+ * functions of fs2moe_router_topk.
+ *   logits [T, E] f32 (as written by fs2moe_router_topk)   topk_idx [T, K]   topk_w, d_w [T, K] f32
+ *   dlogits [T, E] dtype (out)
+ */
+int fs2moe_router_backward(const float* logits, const int32_t* topk_idx, const float* topk_w,
+                           const float* d_w, int32_t T, int32_t E, int32_t K, int32_t score_fn,
+                           int32_t renormalize, int32_t dtype, void* dlogits, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,263 @@
+"""Backward pass on the GPU against ``torch.autograd`` through the CPU oracle in float64.
+
+The oracle's dense formulation follows the reference layer operator for operator (``moe.py:102-157``),
+so differentiating it with autograd gives what the reference's trainer gets (``trainer.py:586-587``).
+Stage tests check each backward entry point on its own; the layer tests check every gradient of the
+module (input, residual, router, expert weights, shared-expert weights) in all routing modes.
+
+Tolerances: gradients are sums of products like the outputs, with one more rounding per intermediate
+(dye, dh, dg/du, dxe are each stored in the activation dtype), so the bf16 bounds are those of the
+forward output widened by sqrt(2): element-wise 3e-2 relative + 6e-2 of the tensor's rms, 1.5e-2 of
+the rms overall; fp32 2e-4 / 2e-4 / 5e-5.  The rms is taken over the entries that are not exactly zero
+in the reference (experts without tokens have zero weight gradients).
+"""
+
+import pytest
+import torch
+
+from fairseq2_amd import _abi
+from fairseq2_amd import workloads as W
+from oracle import moe_oracle as O
+from tests._util import TORCH_DTYPE, build_module
+
+pytestmark = pytest.mark.gpu
+
+GRAD_TOL = {"bf16": (3e-2, 6e-2, 1.5e-2), "fp32": (2e-4, 2e-4, 5e-5)}
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def assert_grad_close(got, ref, dtype, what):
+    got = got.detach().double().cpu().reshape(ref.shape)
+    ref = ref.double()
+    rtol, atol_rel, rms_tol = GRAD_TOL[dtype]
+    # the scale of the entries that are not structurally zero (an expert without tokens has a zero
+    # weight gradient; such blocks would otherwise deflate the scale of the others)
+    nz = ref != 0
+    rms = float(ref[nz].pow(2).mean().sqrt()) if bool(nz.any()) else 0.0
+    assert torch.isfinite(got).all(), f"{what}: non-finite values"
+    err = (got - ref).abs()
+    bound = atol_rel * rms + rtol * ref.abs()
+    worst = float((err / bound).max()) if rms > 0 else float(err.max())
+    err_rms = float(err[nz].pow(2).mean().sqrt()) if rms > 0 else 0.0
+    assert float(err[~nz].max()) <= atol_rel * rms if bool((~nz).any()) else True
+    print(f"  {what}: worst err/bound {worst:.3f}, rms err / rms {err_rms / rms if rms else 0.0:.2e}", flush=True)
+    assert worst <= 1.0, f"{what}: max err/bound {worst:.3f} (rms {rms:.3e})"
+    assert err_rms <= rms_tol * rms, f"{what}: rms error {err_rms:.3e} above {rms_tol} of rms {rms:.3e}"
+
+
+# ------------------------------------------------------------------------------------- stage tests
+def _groups(rows_per_expert, pad=16):
+    counts = torch.tensor(rows_per_expert, dtype=torch.int32)
+    padded = (counts + pad - 1) // pad * pad
+    offsets = torch.zeros(len(rows_per_expert) + 1, dtype=torch.int32)
+    offsets[1:] = torch.cumsum(padded, 0)
+    return counts, offsets
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+@pytest.mark.parametrize("layout", ["in_out", "out_in"])
+@pytest.mark.parametrize("rows,k,n", [([5, 0, 300, 64, 1], 64, 96), ([130, 257], 128, 64), ([40, 3, 0, 77], 72, 40)])
+def test_grouped_gemm_both_orientations(gpu_device, dtype, layout, rows, k, n):
+    _say("grouped_gemm", dtype, layout, rows, k, n)
+    dt = TORCH_DTYPE[dtype]
+    g = torch.Generator().manual_seed(k + n)
+    e = len(rows)
+    counts, offsets = _groups(rows)
+    total = int(offsets[-1])
+    a = torch.randn(total, k, generator=g).to(dt)
+    b = (0.1 * torch.randn(e, k, n, generator=g)).to(dt)
+    stored = b.reshape(e * k, n) if layout == "in_out" else b.transpose(1, 2).contiguous().reshape(e * n, k)
+    dev = gpu_device
+    c = _abi.grouped_gemm(a.to(dev), stored.to(dev), _abi.W_IN_OUT if layout == "in_out" else _abi.W_OUT_IN,
+                          counts.to(dev), offsets.to(dev), e)
+    for ex in range(e):
+        lo, cnt = int(offsets[ex]), int(counts[ex])
+        if cnt:
+            ref = a[lo : lo + cnt].double() @ b[ex].double()
+            assert_grad_close(c[lo : lo + cnt], ref, dtype, f"expert {ex}")
+    # one matrix, all rows
+    d = _abi.grouped_gemm(a.to(dev), stored[: (k if layout == "in_out" else n)].contiguous().to(dev),
+                          _abi.W_IN_OUT if layout == "in_out" else _abi.W_OUT_IN)
+    assert_grad_close(d, a.double() @ b[0].double(), dtype, "dense")
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+@pytest.mark.parametrize("rows,m,n", [([5, 0, 300, 64, 1], 64, 96), ([130, 257], 136, 264), ([33], 8, 8), ([0, 0], 128, 128)])
+def test_grouped_wgrad_matches_torch(gpu_device, dtype, rows, m, n):
+    _say("grouped_wgrad", dtype, rows, m, n)
+    dt = TORCH_DTYPE[dtype]
+    g = torch.Generator().manual_seed(m + n)
+    e = len(rows)
+    counts, offsets = _groups(rows)
+    total = max(int(offsets[-1]), 1)
+    # padding rows hold garbage on purpose: they must not enter the sum
+    a = torch.randn(total, m, generator=g).to(dt)
+    b = torch.randn(total, n, generator=g).to(dt)
+    dev = gpu_device
+    dw = _abi.grouped_wgrad(a.to(dev), b.to(dev), counts.to(dev), offsets.to(dev), e)
+    assert dw.shape == (e * m, n)
+    for ex in range(e):
+        lo, cnt = int(offsets[ex]), int(counts[ex])
+        ref = a[lo : lo + cnt].double().T @ b[lo : lo + cnt].double()
+        got = dw[ex * m : (ex + 1) * m]
+        if cnt == 0:
+            assert float(got.float().abs().max()) == 0.0, "an expert without rows has a zero gradient"
+        else:
+            assert_grad_close(got, ref, dtype, f"expert {ex}")
+    # through a row map, and as one group
+    perm = torch.randperm(total, generator=g).to(torch.int32)
+    dw2 = _abi.grouped_wgrad(a[perm.long()].contiguous().to(dev), b.to(dev), counts.to(dev), offsets.to(dev), e,
+                             a_row_map=torch.argsort(perm).to(torch.int32).to(dev))
+    assert torch.equal(dw2, dw), "row map"
+    one = _abi.grouped_wgrad(a.to(dev), b.to(dev))
+    assert_grad_close(one, a.double().T @ b.double(), dtype, "one group")
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_swiglu_backward_matches_autograd(gpu_device, dtype):
+    dt = TORCH_DTYPE[dtype]
+    gen = torch.Generator().manual_seed(5)
+    g0, u0, dh = (2.0 * torch.randn(77, 40, generator=gen) for _ in range(3))
+    g0, u0, dh = g0.to(dt), u0.to(dt), dh.to(dt)
+    g64, u64 = g0.double().requires_grad_(), u0.double().requires_grad_()
+    h64 = torch.nn.functional.silu(g64) * u64
+    h64.backward(dh.double())
+    h, dg, du = _abi.swiglu_backward(g0.to(gpu_device), u0.to(gpu_device), dh.to(gpu_device))
+    assert_grad_close(h, h64.detach(), dtype, "h")
+    assert_grad_close(dg, g64.grad, dtype, "dg")
+    assert_grad_close(du, u64.grad, dtype, "du")
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_pair_dot(gpu_device, dtype):
+    dt = TORCH_DTYPE[dtype]
+    gen = torch.Generator().manual_seed(6)
+    t, k, d, rows = 50, 3, 72, 400
+    a, a2 = torch.randn(rows, d, generator=gen).to(dt), torch.randn(rows, d, generator=gen).to(dt)
+    b = torch.randn(t, d, generator=gen).to(dt)
+    ar = torch.randint(0, rows, (t, k), generator=gen).to(torch.int32)
+    dev = gpu_device
+    got = _abi.pair_dot(a.to(dev), ar.to(dev), b.to(dev))
+    ref = (a.double()[ar.long()] * b.double()[:, None, :]).sum(-1)
+    torch.testing.assert_close(got.double().cpu(), ref, rtol=1e-5, atol=1e-4)
+    got2 = _abi.pair_dot(a.to(dev), ar.to(dev), b.to(dev), a2=a2.to(dev))
+    ref2 = ((a.float() + a2.float()).double()[ar.long()] * b.double()[:, None, :]).sum(-1)
+    torch.testing.assert_close(got2.double().cpu(), ref2, rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("score_fn,renorm", [("sigmoid", False), ("sigmoid", True), ("softmax", False), ("softmax", True)])
+@pytest.mark.parametrize("e,k", [(16, 4), (128, 8), (8, 8), (200, 3)])
+def test_router_backward_matches_autograd(gpu_device, score_fn, renorm, e, k):
+    gen = torch.Generator().manual_seed(e + k)
+    t = 37
+    logits = (2.0 * torch.randn(t, e, generator=gen)).float()
+    idx = O.topk_lowest_index(logits.double(), k)
+    l64 = logits.double().requires_grad_()
+    w64 = O.combine_weights(l64, idx, score_fn, renorm)
+    d_w = torch.randn(t, k, generator=gen).float()
+    w64.backward(d_w.double())
+    dev = gpu_device
+    code = _abi.SCORE_SOFTMAX if score_fn == "softmax" else _abi.SCORE_SIGMOID
+    dl = _abi.router_backward(logits.to(dev), idx.to(torch.int32).to(dev), w64.detach().float().to(dev),
+                              d_w.to(dev), code, renorm, torch.float32)
+    torch.testing.assert_close(dl.double().cpu(), l64.grad, rtol=2e-4, atol=2e-6)
+
+
+# ------------------------------------------------------------------------------------- whole layer
+MODES = {
+    "reference": W.RoutingMode("sigmoid", False, "input"),
+    "sigmoid_renorm_output": W.RoutingMode("sigmoid", True, "output"),
+    "softmax_renorm_output": W.RoutingMode("softmax", True, "output"),
+    "softmax_input": W.RoutingMode("softmax", False, "input"),
+}
+
+
+def _reference_gradients(wl, grad_out, residual):
+    """float64 autograd through the dense restatement of the reference layer."""
+    s = wl.spec
+    c = lambda t: None if t is None else t.double().clone().requires_grad_(True)  # noqa: E731
+    x, router, gate, up, down = c(wl.x), c(wl.router), c(wl.gate), c(wl.up), c(wl.down)
+    shared = (c(wl.shared_gate), c(wl.shared_up), c(wl.shared_down)) if s.shared else None
+    res = c(residual)
+    out = O.ref_dense_forward(
+        x, router, gate, up, down, s.top_k, shared=shared,
+        router_bias=None if wl.router_bias is None else wl.router_bias.double(),
+        score_fn=s.mode.score_fn, renormalize=s.mode.renormalize, scale_on=s.mode.scale_on,
+    )
+    if res is not None:
+        out = out + res
+    out.backward(grad_out.double())
+    grads = {"x": x.grad, "router": router.grad, "experts.gate_proj": gate.grad,
+             "experts.inner_proj": up.grad, "experts.output_proj": down.grad}
+    if shared is not None:
+        grads.update({"shared_expert.gate_proj.weight": shared[0].grad,
+                      "shared_expert.inner_proj.weight": shared[1].grad,
+                      "shared_expert.output_proj.weight": shared[2].grad})
+    if res is not None:
+        grads["residual"] = res.grad
+    return out.detach(), grads
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize(
+    "mode,shared,zipf,with_residual,shape",
+    [
+        ("reference", False, None, False, dict(tokens=300, model_dim=64, num_experts=8, top_k=2, inner_dim=96)),
+        ("reference", True, None, True, dict(tokens=257, model_dim=128, num_experts=16, top_k=1, inner_dim=64)),
+        ("sigmoid_renorm_output", False, 1.0, False, dict(tokens=200, model_dim=72, num_experts=8, top_k=3, inner_dim=40)),
+        ("softmax_renorm_output", False, 1.2, True, dict(tokens=500, model_dim=128, num_experts=32, top_k=8, inner_dim=192)),
+        ("softmax_input", True, 1.1, False, dict(tokens=130, model_dim=64, num_experts=8, top_k=4, inner_dim=128)),
+    ],
+)
+def test_layer_gradients_match_autograd_of_the_reference(gpu_device, dtype, mode, shared, zipf, with_residual, shape):
+    _say("layer backward", dtype, mode, shared, zipf, with_residual, shape)
+    spec = W.small_spec(dtype=dtype, zipf_s=zipf, shared=shared, mode=MODES[mode], seed=11, **shape)
+    wl = W.make_workload_from_spec(spec)
+    dt = TORCH_DTYPE[dtype]
+    gen = torch.Generator().manual_seed(99)
+    grad_out = torch.randn(wl.x.shape, generator=gen).to(dt).float()
+    residual = torch.randn(wl.x.shape, generator=gen).to(dt).float() if with_residual else None
+    ref_out, ref = _reference_gradients(wl, grad_out, residual)
+
+    m = build_module(wl, gpu_device, tile_m=16).train().requires_grad_(True)
+    x = wl.x.to(dt).to(gpu_device).requires_grad_(True)
+    res = None if residual is None else residual.to(dt).to(gpu_device).requires_grad_(True)
+    out = m(x) if res is None else m(x, residual=res)
+    assert out.requires_grad and out.shape == x.shape
+    with torch.no_grad():
+        plain = m(x.detach()) if res is None else m(x.detach(), residual=res.detach())
+    assert torch.equal(out.detach(), plain), "the training path computes the forward pass's values"
+    out.backward(grad_out.to(dt).to(gpu_device))
+    torch.cuda.synchronize()
+
+    assert_grad_close(x.grad, ref["x"], dtype, "d x")
+    if res is not None:
+        assert torch.equal(res.grad.float().cpu(), grad_out), "the residual's gradient is the output's"
+    for name, p in m.named_parameters():
+        assert p.grad is not None and p.grad.dtype == p.dtype and p.grad.shape == p.shape, name
+        assert_grad_close(p.grad, ref[name], dtype, f"d {name}")
+
+
+def test_frozen_parameters_get_no_gradient_and_unsupported_cases_say_so(gpu_device):
+    wl = W.make_workload_from_spec(W.small_spec(dtype="bf16", tokens=64, num_experts=8, inner_dim=128, seed=3))
+    m = build_module(wl, gpu_device)  # frozen
+    x = wl.x.to(torch.bfloat16).to(gpu_device).requires_grad_(True)
+    out = m(x)
+    out.sum().backward()
+    assert x.grad is not None and all(p.grad is None for p in m.parameters())
+
+    class _Norm:
+        weight, bias, eps, normalized_shape = None, None, 1e-5, (wl.spec.model_dim,)
+
+    with pytest.raises(RuntimeError, match="no backward pass"):
+        m(x, norm=_Norm)
+    m.experts.quantize_fp8_()
+    with pytest.raises(RuntimeError, match="inference format"):
+        m(x)
+    wl10 = W.make_workload_from_spec(W.small_spec(dtype="fp32", tokens=32, num_experts=12, seed=3))
+    m10 = build_module(wl10, gpu_device)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        m10(wl10.x.to(gpu_device).requires_grad_(True))

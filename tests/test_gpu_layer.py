@@ -124,15 +124,22 @@ def test_deterministic_and_tile_size_independent(gpu_device):
         assert torch.equal(o, outs[0]), "output must not depend on the run or on the padding granularity"
 
 
-def test_forward_only_contract(gpu_device):
+def test_gradient_and_device_contract(gpu_device):
+    # With parameters that require a gradient the call goes through the differentiable function (its
+    # gradients are checked in tests/test_gpu_backward.py) and returns the same values; the stand-alone
+    # expert modules are forward-only and say so.
     wl = W.make_workload_from_spec(W.small_spec(tokens=8, dtype="bf16"))
     m = build_module(wl, gpu_device)
     x = wl.x.to(torch.bfloat16).to(gpu_device)
-    m.requires_grad_(True)
-    with pytest.raises(RuntimeError, match="forward-only"):
-        m(x)
     with torch.no_grad():
-        m(x)
+        want = m(x)
+    m.requires_grad_(True)
+    got = m(x)
+    assert got.requires_grad and torch.equal(got.detach(), want)
+    with torch.no_grad():
+        assert not m(x).requires_grad
+    with pytest.raises(RuntimeError, match="forward-only"):
+        m.experts(x.reshape(1, -1, x.shape[-1]).expand(8, -1, -1).contiguous())
     with pytest.raises(RuntimeError, match="GPU only"):
         m.requires_grad_(False)(x.cpu())
 
