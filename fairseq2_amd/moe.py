@@ -6,8 +6,10 @@
 (``models/transformer_lm/decoder_layer.py:194``) can call it unchanged and a
 reference checkpoint loads with ``load_state_dict``.  The forward pass is four
 device stages behind a C ABI: router + top-k, dispatch, grouped SwiGLU experts
-(+ the optional shared expert) and combine.  It is forward-only and runs on the
-GPU only; there is no torch-operator fallback.
+(+ the optional shared expert) and combine.  It runs on the GPU only; there is no
+torch-operator fallback.  With inputs or parameters that require a gradient the
+layer runs as one ``torch.autograd.Function`` whose backward pass uses the same
+library (:mod:`fairseq2_amd.autograd`).
 
 Keyword-only extensions (defaults reproduce the reference):
 
@@ -43,7 +45,7 @@ class FeedForwardNetwork(Module, ABC):
 def _require_forward_only(*tensors: Tensor | None) -> None:
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
         raise RuntimeError(
-            "fairseq2_amd.MoE is forward-only: call it under torch.no_grad() / "
+            "this fairseq2_amd module is forward-only: call it under torch.no_grad() / "
             "torch.inference_mode(), or freeze the module with requires_grad_(False)"
         )
 
