@@ -159,17 +159,23 @@ def cpu_baseline(wl, seconds: float) -> dict:
 
     probe_n = min(64, spec.num_tokens)
     run(probe_n)  # warm-up (thread pool, kernels selection)
-    per_tok = run(probe_n) / probe_n
-    n = int(max(probe_n, min(spec.num_tokens, seconds / max(per_tok, 1e-9))))
-    n = min(spec.num_tokens, max(probe_n, (n // 64) * 64 or probe_n))
-    dt_s = run(n)
+    # Grow the sample until one pass takes about `seconds`: small samples run at a lower rate (the
+    # per-expert matrix products are too small to use the cores), so a size extrapolated from the
+    # probe alone would fall well short of the target time.
+    n, dt_s = probe_n, run(probe_n)
+    for _ in range(3):
+        if dt_s >= 0.6 * seconds or n >= spec.num_tokens:
+            break
+        want = int(n * min(16.0, 0.9 * seconds / max(dt_s, 1e-9)))
+        n = min(spec.num_tokens, max(n + 64, want // 64 * 64))
+        dt_s = run(n)
     return {
         "value": n / dt_s,
         "unit": "tokens/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
         "sample": f"dense reference formulation in {str(dt).replace('torch.', '')} on the first {n} of "
-                  f"{spec.num_tokens} tokens, one timed pass of {dt_s:.2f} s after a warm-up",
+                  f"{spec.num_tokens} tokens, one timed pass of {dt_s:.2f} s (after shorter passes that sized it)",
     }
 
 

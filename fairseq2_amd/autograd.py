@@ -31,80 +31,91 @@ from torch import Tensor
 from fairseq2_amd import _abi
 
 
+def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg):
+    """The staged forward pass; returns ``(out, saved)`` with what :func:`backward_from` needs."""
+    e, k, tile_m = cfg["num_experts"], cfg["top_k"], cfg["tile_m"]
+    score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
+    idx, w, logits = _abi.router_topk(x, router, cfg["router_bias"], k, score_fn, renorm, want_logits=True)
+    disp = _abi.dispatch(idx, w, x, e, tile_m, scale_input, gather=True)
+    ye, _ = _abi.grouped_swiglu(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
+    base = _abi.dense_swiglu(x, sg, su, sd) if sg is not None else None
+    out = _abi.combine(ye, disp.inv_perm, idx, w, base, not scale_input, out=base, residual=residual)
+    return out, (idx, w, logits, disp.counts, disp.offsets, disp.inv_perm, disp.xe, ye)
+
+
+def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
+    """Gradients ``(dx, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd)`` (None where ``need`` -- in
+    that order -- says so) from the output gradient and the intermediates of :func:`forward_saving`."""
+    idx, w, logits, counts, offsets, inv_perm, xe, ye = saved
+    e, tile_m = cfg["num_experts"], cfg["tile_m"]
+    score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
+    dout = dout.contiguous()
+    IN_OUT, OUT_IN = _abi.W_IN_OUT, _abi.W_OUT_IN
+    grp = dict(counts=counts, offsets=offsets, num_experts=e)
+
+    # output gradients in expert order (times the combine weight when it scales the output);
+    # the permutation is the forward pass's: dispatch is deterministic
+    dye = _abi.dispatch(idx, w, dout, e, tile_m, not scale_input, gather=True).xe
+    dh = _abi.grouped_gemm(dye, wd, OUT_IN, **grp)
+    g = _abi.grouped_gemm(xe, wg, IN_OUT, **grp)
+    u = _abi.grouped_gemm(xe, wu, IN_OUT, **grp)
+    h, dg, du = _abi.swiglu_backward(g, u, dh)
+    d_wd = _abi.grouped_wgrad(h, dye, **grp) if need[4] else None
+    d_wg = _abi.grouped_wgrad(xe, dg, **grp) if need[2] else None
+    d_wu = _abi.grouped_wgrad(xe, du, **grp) if need[3] else None
+    dxe_g = _abi.grouped_gemm(dg, wg, OUT_IN, **grp)
+    dxe_u = _abi.grouped_gemm(du, wu, OUT_IN, **grp)
+
+    # combine weights -> logits -> router and x
+    if scale_input:
+        d_w = _abi.pair_dot(dxe_g, inv_perm, x, a2=dxe_u)
+    else:
+        d_w = _abi.pair_dot(ye, inv_perm, dout)
+    dl = _abi.router_backward(logits, idx, w, d_w, score_fn, renorm, x.dtype)
+    d_router = _abi.grouped_wgrad(x, dl) if need[1] else None
+    dx_parts = [_abi.grouped_gemm(dl, router, OUT_IN)] if need[0] else []
+
+    d_sg = d_su = d_sd = None
+    if sg is not None:
+        dh_s = _abi.grouped_gemm(dout, sd, IN_OUT)
+        g_s = _abi.grouped_gemm(x, sg, OUT_IN)
+        u_s = _abi.grouped_gemm(x, su, OUT_IN)
+        h_s, dg_s, du_s = _abi.swiglu_backward(g_s, u_s, dh_s)
+        d_sd = _abi.grouped_wgrad(dout, h_s) if need[7] else None
+        d_sg = _abi.grouped_wgrad(dg_s, x) if need[5] else None
+        d_su = _abi.grouped_wgrad(du_s, x) if need[6] else None
+        if need[0]:
+            dx_parts += [_abi.grouped_gemm(dg_s, sg, IN_OUT), _abi.grouped_gemm(du_s, su, IN_OUT)]
+
+    dx = None
+    if need[0]:
+        # dx[t] = sum_k s_k dxe[row(t, k)] + the dense terms (at most three: router, and two of the
+        # shared expert): two scatter passes, one per half of dxe, each starting from up to two dense
+        # rows (the kernel's base and residual operands), everything summed in f32
+        dense = dx_parts + [None] * (3 - len(dx_parts))
+        t1 = _abi.combine(dxe_g, inv_perm, idx, w, dense[0], scale_input, residual=dense[1])
+        dx = _abi.combine(dxe_u, inv_perm, idx, w, t1, scale_input, out=t1, residual=dense[2])
+    return dx, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd
+
+
 class MoEFunction(torch.autograd.Function):
     """``forward(x, residual, router, wg, wu, wd, sg, su, sd, cfg)``; ``cfg`` carries the integers."""
 
     @staticmethod
     def forward(ctx, x, residual, router, wg, wu, wd, sg, su, sd, cfg):  # noqa: D102
-        e, k, tile_m = cfg["num_experts"], cfg["top_k"], cfg["tile_m"]
-        score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
-        idx, w, logits = _abi.router_topk(x, router, cfg["router_bias"], k, score_fn, renorm, want_logits=True)
-        disp = _abi.dispatch(idx, w, x, e, tile_m, scale_input, gather=True)
-        ye, _ = _abi.grouped_swiglu(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
-        base = _abi.dense_swiglu(x, sg, su, sd) if sg is not None else None
-        out = _abi.combine(ye, disp.inv_perm, idx, w, base, not scale_input, out=base, residual=residual)
+        out, saved = forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg)
         ctx.cfg = cfg
         ctx.has_residual = residual is not None
-        ctx.has_shared = sg is not None
-        ctx.save_for_backward(x, router, wg, wu, wd, sg, su, sd, idx, w, logits, disp.counts,
-                              disp.offsets, disp.inv_perm, disp.xe, ye)
+        ctx.save_for_backward(x, router, wg, wu, wd, sg, su, sd, *saved)
         return out
 
     @staticmethod
     @torch.no_grad()
     def backward(ctx, dout):  # noqa: D102
-        (x, router, wg, wu, wd, sg, su, sd, idx, w, logits, counts, offsets, inv_perm, xe,
-         ye) = ctx.saved_tensors
-        cfg = ctx.cfg
-        e, tile_m = cfg["num_experts"], cfg["tile_m"]
-        score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
-        need = ctx.needs_input_grad
-        dout = dout.contiguous()
-        IN_OUT, OUT_IN = _abi.W_IN_OUT, _abi.W_OUT_IN
-        grp = dict(counts=counts, offsets=offsets, num_experts=e)
-
-        # output gradients in expert order (times the combine weight when it scales the output);
-        # the permutation is the forward pass's: dispatch is deterministic
-        dye = _abi.dispatch(idx, w, dout, e, tile_m, not scale_input, gather=True).xe
-        dh = _abi.grouped_gemm(dye, wd, OUT_IN, **grp)
-        g = _abi.grouped_gemm(xe, wg, IN_OUT, **grp)
-        u = _abi.grouped_gemm(xe, wu, IN_OUT, **grp)
-        h, dg, du = _abi.swiglu_backward(g, u, dh)
-        d_wd = _abi.grouped_wgrad(h, dye, **grp) if need[5] else None
-        d_wg = _abi.grouped_wgrad(xe, dg, **grp) if need[3] else None
-        d_wu = _abi.grouped_wgrad(xe, du, **grp) if need[4] else None
-        dxe_g = _abi.grouped_gemm(dg, wg, OUT_IN, **grp)
-        dxe_u = _abi.grouped_gemm(du, wu, OUT_IN, **grp)
-
-        # combine weights -> logits -> router and x
-        if scale_input:
-            d_w = _abi.pair_dot(dxe_g, inv_perm, x, a2=dxe_u)
-        else:
-            d_w = _abi.pair_dot(ye, inv_perm, dout)
-        dl = _abi.router_backward(logits, idx, w, d_w, score_fn, renorm, x.dtype)
-        d_router = _abi.grouped_wgrad(x, dl) if need[2] else None
-        dx_parts = [_abi.grouped_gemm(dl, router, OUT_IN)] if need[0] else []
-
-        d_sg = d_su = d_sd = None
-        if ctx.has_shared:
-            dh_s = _abi.grouped_gemm(dout, sd, IN_OUT)
-            g_s = _abi.grouped_gemm(x, sg, OUT_IN)
-            u_s = _abi.grouped_gemm(x, su, OUT_IN)
-            h_s, dg_s, du_s = _abi.swiglu_backward(g_s, u_s, dh_s)
-            d_sd = _abi.grouped_wgrad(dout, h_s) if need[8] else None
-            d_sg = _abi.grouped_wgrad(dg_s, x) if need[6] else None
-            d_su = _abi.grouped_wgrad(du_s, x) if need[7] else None
-            if need[0]:
-                dx_parts += [_abi.grouped_gemm(dg_s, sg, IN_OUT), _abi.grouped_gemm(du_s, su, IN_OUT)]
-
-        dx = None
-        if need[0]:
-            # dx[t] = sum_k s_k dxe[row(t, k)] + the dense terms (at most three: router, and two of
-            # the shared expert): two scatter passes, one per half of dxe, each starting from up to
-            # two dense rows (the kernel's base and residual operands), everything summed in f32
-            dense = dx_parts + [None] * (3 - len(dx_parts))
-            t1 = _abi.combine(dxe_g, inv_perm, idx, w, dense[0], scale_input, residual=dense[1])
-            dx = _abi.combine(dxe_u, inv_perm, idx, w, t1, scale_input, out=t1, residual=dense[2])
-        d_res = dout if ctx.has_residual and need[1] else None
+        x, router, wg, wu, wd, sg, su, sd, *saved = ctx.saved_tensors
+        n = ctx.needs_input_grad
+        need = (n[0], n[2], n[3], n[4], n[5], n[6], n[7], n[8])
+        dx, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd = backward_from(
+            x, router, wg, wu, wd, sg, su, sd, tuple(saved), ctx.cfg, dout, need)
+        d_res = dout if ctx.has_residual and n[1] else None
         return dx, d_res, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd, None
-

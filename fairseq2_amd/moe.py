@@ -97,13 +97,17 @@ class GroupedExpertNetwork(ExpertNetwork):
         dtype: torch.dtype | None = None,
     ) -> None:
         super().__init__(num_experts, model_dim, inner_dim)
-        if activation is not None and not isinstance(activation, nn.SiLU):
-            raise NotImplementedError("the fused expert kernels implement the SiLU gate only")
         kw = dict(device=device, dtype=dtype)
         self.gate_proj = Parameter(torch.empty((num_experts * model_dim, inner_dim), **kw))
         self.inner_proj = Parameter(torch.empty((num_experts * model_dim, inner_dim), **kw))
         self.output_proj = Parameter(torch.empty((num_experts * inner_dim, model_dim), **kw))
-        self.activation = nn.SiLU()
+        # Any module, as in the reference (experts.py:84-87).  The fused kernels implement the SiLU
+        # gate; another activation runs between plain grouped GEMMs of the same library.
+        self.activation = activation if activation is not None else nn.SiLU()
+
+    @property
+    def has_fused_gate(self) -> bool:
+        return isinstance(self.activation, nn.SiLU)
 
     # ---- fp8 (e4m3) weights: derived, non-persistent buffers next to the Parameters ----------------
     # Stored as integers (codes as uint8, scales as the int32 bit patterns of their f32 values) so
@@ -187,6 +191,8 @@ class GroupedExpertNetwork(ExpertNetwork):
     def fuses_gather(self, act_dtype: torch.dtype, max_rows: int = 0) -> bool:
         """Whether :meth:`forward_rows` can read ``max_rows`` rows through a row map from the token
         matrix (no gathered copy needed)."""
+        if not self.has_fused_gate:
+            return False
         if self.has_fp8_weights:
             return _abi.fuses_gather(self.model_dim, self.inner_dim, act_dtype, torch.float8_e4m3fn)
         # the bf16 kernel addresses its activation matrices with 32-bit byte offsets
@@ -199,6 +205,14 @@ class GroupedExpertNetwork(ExpertNetwork):
     ) -> Tensor:
         """Runs every expert on its block of rows of ``xe`` (rows, D); with ``row_map``, row ``r``
         is ``xe[row_map[r]]`` and ``xe`` is the token matrix."""
+        if not self.has_fused_gate:
+            # experts.py:107-112 with the module's own activation between the library's GEMMs
+            if self.has_fp8_weights or row_map is not None:
+                raise NotImplementedError("e4m3 weights and the fused gather need the SiLU gate")
+            grp = dict(counts=counts, offsets=offsets, num_experts=self.num_local_experts)
+            h = self.activation(_abi.grouped_gemm(xe, self.gate_proj.detach(), _abi.W_IN_OUT, **grp))
+            h = (h * _abi.grouped_gemm(xe, self.inner_proj.detach(), _abi.W_IN_OUT, **grp)).to(xe.dtype)
+            return _abi.grouped_gemm(h.contiguous(), self.output_proj.detach(), _abi.W_IN_OUT, **grp)
         if self.has_fp8_weights:
             ye, _ = _abi.grouped_swiglu(
                 xe, counts, offsets, self.gate_q, self.inner_q, self.output_q,
@@ -411,23 +425,28 @@ class MoE(FeedForwardNetwork):
         seqs = self._autocast(seqs)
         if residual is not None:
             residual = self._autocast(residual)
-        if torch.is_grad_enabled() and any(
+        wants_grad = torch.is_grad_enabled() and any(
             t is not None and t.requires_grad for t in (seqs, residual, *self.parameters())
-        ):
+        )
+        if wants_grad and not torch.compiler.is_compiling():
             return self._differentiable(seqs, residual, norm)
-        x = self._checked_rows(seqs)
+        # (while a compiler traces the call, training goes through the registered operator below,
+        # which carries its own autograd formula)
+        x = self._checked_rows(seqs, allow_grad=wants_grad)
         norm_args = self._norm_args(norm, x)
         res = None
         if residual is not None:
             if residual.shape != seqs.shape or residual.dtype != seqs.dtype:
                 raise ValueError("residual must have the shape and dtype of seqs")
             _require_device(residual)
-            _require_forward_only(residual)
+            if not wants_grad:
+                _require_forward_only(residual)
             res = residual.reshape(-1, seqs.shape[-1]).contiguous()
         if x.shape[0] == 0:
             return torch.empty_like(seqs)
         ex, se = self.experts, self.shared_expert
-        if type(ex) is GroupedExpertNetwork and (se is None or type(se) is GLUFeedForwardNetwork):
+        if (type(ex) is GroupedExpertNetwork and ex.has_fused_gate
+                and (se is None or type(se) is GLUFeedForwardNetwork)):
             return self._single_call(x, res, norm_args).view(seqs.shape)
         return self._stages(x, res, norm_args)[0].view(seqs.shape)
 
@@ -442,6 +461,8 @@ class MoE(FeedForwardNetwork):
             why = "the normalisation fused into the router has no backward pass (normalise outside the layer)"
         elif type(ex) is not GroupedExpertNetwork or (se is not None and type(se) is not GLUFeedForwardNetwork):
             why = "only GroupedExpertNetwork experts and a GLUFeedForwardNetwork shared expert are differentiated"
+        elif not ex.has_fused_gate:
+            why = "only the SiLU gate is differentiated"
         elif ex.has_fp8_weights:
             why = "e4m3 expert weights are an inference format"
         elif ex.num_local_experts % 8:
@@ -504,7 +525,6 @@ class MoE(FeedForwardNetwork):
             weight = weight.detach().contiguous()
         return weight, float(norm.eps)
 
-    @torch.no_grad()
     def _single_call(self, x: Tensor, residual: Tensor | None = None, norm=None) -> Tensor:
         """The layer through the library's whole-layer entry point: one call, one workspace
         allocation (same kernels and results as :meth:`_stages`)."""
@@ -520,9 +540,14 @@ class MoE(FeedForwardNetwork):
             shared = (se.gate_proj.weight.detach(), se.inner_proj.weight.detach(), se.output_proj.weight.detach())
         if torch.compiler.is_compiling():
             # under torch.compile the call goes through the registered operator, which the tracer
-            # can represent (it cannot look through ctypes)
+            # can represent (it cannot look through ctypes); it is given the parameters themselves,
+            # so that its autograd formula reaches them when the trace is one of a training step
+            if not ex.has_fp8_weights:
+                weights = (ex.gate_proj, ex.inner_proj, ex.output_proj)
+            if se is not None:
+                shared = (se.gate_proj.weight, se.inner_proj.weight, se.output_proj.weight)
             return torch.ops.fairseq2_amd.moe_forward(
-                x, self.router.detach(), self.router_bias, *weights, *(scales or (None, None, None)),
+                x, self.router, self.router_bias, *weights, *(scales or (None, None, None)),
                 *(shared or (None, None, None)), residual, None if norm is None else norm[0],
                 ex.num_local_experts, self.top_k, self.tile_m, _SCORE_FNS[self.score_fn],
                 self.renormalize, self.scale_on == "input", norm is not None,

@@ -7,8 +7,11 @@ being traced: the operator carries a shape-only ("fake") implementation for the 
 one, the whole-layer entry point of the library, for the GPU.  Outside a trace the module calls the
 library directly (an operator dispatch costs more host time than a decode-sized layer takes).
 
-Forward only: no autograd formula is registered, and the module refuses inputs that require a
-gradient before it gets here.
+Training under ``torch.compile``: the operator has an autograd formula, a second registered operator
+``torch.ops.fairseq2_amd.moe_backward`` that recomputes the forward pass's intermediates (routing,
+gathered rows, expert outputs) and runs the backward kernels of :mod:`fairseq2_amd.autograd`; a
+compiled layer therefore stays one graph in training as well, for the recomputation's price.  Eager
+training does not pay it (the module keeps the intermediates of its own forward pass).
 """
 
 from __future__ import annotations
@@ -60,3 +63,78 @@ def moe_forward(
 @moe_forward.register_fake
 def _moe_forward_fake(x, *args, **kwargs):
     return torch.empty_like(x)
+
+
+@torch.library.custom_op("fairseq2_amd::moe_backward", mutates_args=(), device_types="cuda")
+def moe_backward(
+    grad_out: Tensor,
+    x: Tensor,
+    router: Tensor,
+    router_bias: Optional[Tensor],
+    w_gate: Tensor,
+    w_up: Tensor,
+    w_down: Tensor,
+    shared_gate: Optional[Tensor],
+    shared_up: Optional[Tensor],
+    shared_down: Optional[Tensor],
+    num_experts: int,
+    top_k: int,
+    tile_m: int,
+    score_fn: int,
+    renormalize: bool,
+    scale_input: bool,
+) -> list[Tensor]:
+    """Gradients of ``moe_forward`` for ``x``, ``router``, the three expert weights and (when given)
+    the three shared-expert weights, in that order (5 or 8 tensors)."""
+    from fairseq2_amd.autograd import backward_from, forward_saving
+
+    cfg = dict(num_experts=num_experts, top_k=top_k, tile_m=tile_m, score_fn=score_fn,
+               renormalize=renormalize, scale_input=scale_input, router_bias=router_bias)
+    _, saved = forward_saving(x, None, router, w_gate, w_up, w_down, shared_gate, shared_up,
+                              shared_down, cfg)
+    grads = backward_from(x, router, w_gate, w_up, w_down, shared_gate, shared_up, shared_down,
+                          saved, cfg, grad_out, (True,) * 8)
+    return [g for g in grads if g is not None]
+
+
+@moe_backward.register_fake
+def _moe_backward_fake(grad_out, x, router, router_bias, w_gate, w_up, w_down, shared_gate,
+                       shared_up, shared_down, *ints):
+    out = [torch.empty_like(t) for t in (x, router, w_gate, w_up, w_down)]
+    if shared_gate is not None:
+        out += [torch.empty_like(t) for t in (shared_gate, shared_up, shared_down)]
+    return out
+
+
+def _setup_context(ctx, inputs, output):
+    (x, router, router_bias, w_gate, w_up, w_down, s_gate, s_up, s_down, shared_gate, shared_up,
+     shared_down, residual, norm_weight, num_experts, top_k, tile_m, score_fn, renormalize,
+     scale_input, normed, norm_eps) = inputs
+    if s_gate is not None or normed:
+        ctx.unsupported = "e4m3 weights and the fused normalisation are forward-only"
+        return
+    if num_experts % 8:
+        ctx.unsupported = "the router's backward kernels need a number of experts that is a multiple of 8"
+        return
+    ctx.unsupported = None
+    ctx.ints = (num_experts, top_k, tile_m, score_fn, renormalize, scale_input)
+    ctx.has_residual = residual is not None
+    ctx.has_shared = shared_gate is not None
+    ctx.save_for_backward(x, router, router_bias, w_gate, w_up, w_down, shared_gate, shared_up, shared_down)
+
+
+def _backward(ctx, grad_out):
+    if ctx.unsupported is not None:
+        raise RuntimeError(f"fairseq2_amd::moe_forward: {ctx.unsupported}")
+    x, router, router_bias, w_gate, w_up, w_down, sg, su, sd = ctx.saved_tensors
+    grads = torch.ops.fairseq2_amd.moe_backward(
+        grad_out.contiguous(), x, router, router_bias, w_gate, w_up, w_down, sg, su, sd, *ctx.ints)
+    dx, d_router, d_wg, d_wu, d_wd = grads[:5]
+    d_sg, d_su, d_sd = grads[5:8] if ctx.has_shared else (None, None, None)
+    d_res = grad_out if ctx.has_residual else None
+    # one entry per argument of moe_forward
+    return (dx, d_router, None, d_wg, d_wu, d_wd, None, None, None, d_sg, d_su, d_sd, d_res, None,
+            None, None, None, None, None, None, None, None)
+
+
+moe_forward.register_autograd(_backward, setup_context=_setup_context)

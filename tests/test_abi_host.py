@@ -199,8 +199,11 @@ def test_extension_options_are_validated():
             M.MoE(64, 64, False, 1000, 1.0, 1, **kw)
         with pytest.raises(ValueError, match="multiples of 8"):
             M.MoE(60, 64, False, 4, 1.0, 1, **kw)
-        with pytest.raises(NotImplementedError, match="SiLU"):
-            M.MoE(64, 64, False, 4, 1.0, 1, moe_activation=torch.nn.GELU(), **kw)
+        # any activation module is accepted, as in the reference (experts.py:84-87); only the SiLU
+        # gate runs fused
+        g = M.MoE(64, 64, False, 4, 1.0, 1, moe_activation=torch.nn.GELU(), **kw)
+        assert isinstance(g.experts.activation, torch.nn.GELU) and not g.experts.has_fused_gate
+        assert M.MoE(64, 64, False, 4, 1.0, 1, **kw).experts.has_fused_gate
         m = M.MoE(64, 64, False, 4, 1.0, 1, router_bias=True, **kw)
     assert "router_bias" in m.state_dict()
 

@@ -261,3 +261,34 @@ def test_frozen_parameters_get_no_gradient_and_unsupported_cases_say_so(gpu_devi
     m10 = build_module(wl10, gpu_device)
     with pytest.raises(RuntimeError, match="multiple of 8"):
         m10(wl10.x.to(gpu_device).requires_grad_(True))
+
+
+@pytest.mark.parametrize("shared,with_residual", [(False, False), (True, True)])
+def test_training_step_under_torch_compile(gpu_device, shared, with_residual):
+    """A compiled layer in training mode (transformer_lm/compiler.py:14-17 wraps layers that the
+    trainer then differentiates): the registered operator carries an autograd formula, so the trace is
+    one graph, and its gradients are those of the eager training path (same kernels: bit-equal)."""
+    _say("compiled training step", shared, with_residual)
+    spec = W.small_spec(tokens=200, model_dim=128, num_experts=8, top_k=2, inner_dim=64, dtype="bf16",
+                        shared=shared, mode=W.RoutingMode("softmax", True, "output"), zipf_s=1.0, seed=21)
+    wl = W.make_workload_from_spec(spec)
+    gen = torch.Generator().manual_seed(5)
+    g = torch.randn(wl.x.shape, generator=gen).to(torch.bfloat16).to(gpu_device)
+
+    def grads(compiled):
+        m = build_module(wl, gpu_device).train().requires_grad_(True)
+        x = wl.x.to(torch.bfloat16).to(gpu_device).requires_grad_(True)
+        fn = (lambda t: m(t, residual=t)) if with_residual else (lambda t: m(t))  # noqa: E731
+        if compiled:
+            fn = torch.compile(fn, backend="aot_eager", fullgraph=True)
+        out = fn(x)
+        out.backward(g)
+        torch.cuda.synchronize()
+        return out.detach(), x.grad, {n: p.grad for n, p in m.named_parameters()}
+
+    out_e, dx_e, dp_e = grads(False)
+    out_c, dx_c, dp_c = grads(True)
+    assert torch.equal(out_c, out_e)
+    assert torch.equal(dx_c, dx_e)
+    for n in dp_e:
+        assert dp_c[n] is not None and torch.equal(dp_c[n], dp_e[n]), n

@@ -124,6 +124,37 @@ def test_deterministic_and_tile_size_independent(gpu_device):
         assert torch.equal(o, outs[0]), "output must not depend on the run or on the padding granularity"
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+@pytest.mark.parametrize("shared", [False, True])
+def test_other_expert_activation(gpu_device, dtype, shared):
+    """``moe_activation`` other than SiLU (the reference takes any module, ``llama4/moe.py:44``,
+    ``experts.py:84-87``): the experts then run as plain grouped GEMMs of the library around the
+    module's own activation.  Checked against the same formula in float64."""
+    act = torch.nn.GELU(approximate="tanh")
+    spec = W.small_spec(tokens=300, model_dim=128, num_experts=8, top_k=2, inner_dim=192, dtype=dtype,
+                        shared=shared, seed=5)
+    wl = W.make_workload_from_spec(spec)
+    m = build_module(wl, gpu_device)
+    m.experts.activation = act
+    assert not m.experts.has_fused_gate
+    x = wl.x.to(TORCH_DTYPE[dtype]).to(gpu_device)
+    with torch.no_grad():
+        out = m(x)
+    _, idx, w = oracle_routing(wl)
+    t, d, e, f = spec.num_tokens, spec.model_dim, spec.num_experts, spec.inner_dim
+    xd = wl.x.reshape(t, d).double()
+    ref = O.shared_glu(xd, wl.shared_gate.double(), wl.shared_up.double(), wl.shared_down.double()) if shared else torch.zeros(t, d, dtype=torch.float64)
+    for tok in range(t):
+        for j in range(spec.top_k):
+            ex = int(idx[tok, j])
+            u = xd[tok] * w[tok, j]
+            h = act(u @ wl.gate.double()[ex * d : (ex + 1) * d]) * (u @ wl.up.double()[ex * d : (ex + 1) * d])
+            ref[tok] += h @ wl.down.double()[ex * f : (ex + 1) * f]
+    assert_output_close(out, ref, dtype, "GELU-gated experts")
+    with pytest.raises(RuntimeError, match="SiLU gate is differentiated"):
+        m.requires_grad_(True)(x)
+
+
 def test_gradient_and_device_contract(gpu_device):
     # With parameters that require a gradient the call goes through the differentiable function (its
     # gradients are checked in tests/test_gpu_backward.py) and returns the same values; the stand-alone

@@ -28,3 +28,16 @@ def test_operator_is_registered_with_a_shape_only_implementation():
 def test_operator_has_no_cpu_implementation():
     with pytest.raises(NotImplementedError):
         torch.ops.fairseq2_amd.moe_forward(*[a.zero_() if isinstance(a, torch.Tensor) else a for a in _args("cpu")])
+
+
+def test_backward_operator_is_registered_with_a_shape_only_implementation():
+    op = torch.ops.fairseq2_amd.moe_backward
+    with FakeTensorMode():
+        a = _args("cuda")
+        x, router, _, w_in, _, w_out = a[:6]
+        grads = op(torch.empty_like(x), x, router, None, w_in, w_in, w_out, None, None, None, 8, 2, 16, 0, False, True)
+        assert [g.shape for g in grads] == [x.shape, router.shape, w_in.shape, w_in.shape, w_out.shape]
+        sg = torch.empty(32, 64, device="cuda", dtype=torch.bfloat16)
+        sd = torch.empty(64, 32, device="cuda", dtype=torch.bfloat16)
+        grads = op(torch.empty_like(x), x, router, None, w_in, w_in, w_out, sg, sg, sd, 8, 2, 16, 0, False, True)
+        assert len(grads) == 8 and grads[7].shape == sd.shape
