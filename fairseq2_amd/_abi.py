@@ -90,10 +90,11 @@ _PROTOTYPES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32,
          c_int64, c_int32, c_void_p, c_void_p],
     ),
+    "fs2moe_grouped_wgrad_workspace_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int64]),
     "fs2moe_grouped_wgrad": (
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int64,
-         c_int32, c_void_p, c_void_p],
+         c_int32, c_void_p, c_void_p, c_int64, c_void_p],
     ),
     "fs2moe_swiglu_backward": (
         c_int32,
@@ -543,9 +544,11 @@ def grouped_wgrad(
     elif a.shape[0] != rows:
         raise ValueError("a and b must have the same number of rows")
     dw = torch.empty((e * m, n), dtype=a.dtype, device=a.device)
+    ws_bytes = lib.fs2moe_grouped_wgrad_workspace_bytes(int(counts is not None), m, n, rows)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes > 0 else None
     rc = lib.fs2moe_grouped_wgrad(
         _ptr(a), _ptr(a_row_map), _ptr(b), _ptr(counts), _ptr(offsets), e, m, n, rows,
-        dtype_code(a.dtype), _ptr(dw), _stream(),
+        dtype_code(a.dtype), _ptr(dw), _ptr(ws), max(ws_bytes, 0), _stream(),
     )
     _check(rc, "fs2moe_grouped_wgrad")
     return dw

@@ -16,77 +16,114 @@
 namespace fs2moe {
 
 // ---------------------------------------------------------------------------------- weight gradient
-// C_e [M, N] = sum over the rows r of expert e of A[r, :M]^T B[r, :N].  A block owns a 128 x 128 tile
-// of one expert's gradient and walks the expert's rows 32 at a time: both chunks go to LDS as they
-// lie in memory (row = contraction index, columns contiguous) and come back through the transposing
-// LDS read (bf16) or as single floats (f32), each already in MFMA operand order.  Rows past the
-// expert's count are zero-filled, experts without rows get a zero gradient.
+// C_e [M, N] = sum over the rows r of expert e of A[r, :M]^T B[r, :N].  A block of 8 waves owns a
+// 256 x 256 tile of one expert's gradient (a wave 128 x 64: 4 x 2 MFMA tiles) and walks the expert's
+// rows RK at a time (32 for bf16, 16 for f32).  Both chunks go to LDS as they lie in memory (row =
+// contraction index, columns contiguous) and come back through the transposing LDS read (bf16) or
+// as single floats (f32), each already in MFMA operand order.  LDS holds two chunks: while one is
+// multiplied the next is written from registers and the one after that is on its way from memory,
+// so there is one barrier per chunk.  Rows past the expert's count are zero-filled, experts without
+// rows get a zero gradient.
 namespace wgk {
-constexpr int TM = 128, TN = 128, RK = 32;
+constexpr int TM = 256, TN = 256, WAVES = 8;
+constexpr int SMEM_BYTES = 65536;  // two chunks of both operands
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void grouped_wgrad_kernel(
+__global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
     const T* __restrict__ A, const int32_t* __restrict__ a_map, int lda, const T* __restrict__ B,
-    int ldb, T* __restrict__ C, int M, int N, Groups g, int m_tiles, int n_tiles) {
+    int ldb, T* __restrict__ C, int M, int N, Groups g, int m_tiles, int n_tiles, int seg_rows,
+    float* __restrict__ partial) {
   using namespace wgk;
   constexpr bool BF16 = sizeof(T) == 2;
+  constexpr int RK = BF16 ? 32 : 16;              // rows per chunk
   constexpr int VEC = 16 / sizeof(T);             // elements per 16-byte chunk
-  constexpr int ROW_CHUNKS = TM / VEC;            // chunks per LDS row (16 or 32)
-  constexpr int PER_THREAD = RK * ROW_CHUNKS / 256;  // chunks per thread and operand (2 or 4)
-  constexpr int ROWB = TM * sizeof(T);            // bytes per LDS row
-  __shared__ __attribute__((aligned(16))) uint8_t sA[RK * ROWB];
-  __shared__ __attribute__((aligned(16))) uint8_t sB[RK * ROWB];
+  constexpr int ROW_CHUNKS = TM / VEC;            // 16-byte chunks per LDS row (32 or 64)
+  constexpr int PER_THREAD = RK * ROW_CHUNKS / (WAVES * 64);  // chunks per thread and operand (2)
+  constexpr int ROWB = TM * sizeof(T);            // bytes per LDS row (512 or 1024)
+  constexpr int OPB = RK * ROWB;                  // bytes per operand chunk (16 KB)
+  static_assert(4 * OPB == SMEM_BYTES, "two chunks of two operands");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int per_e = m_tiles * n_tiles;
-  const int e = blockIdx.x / per_e;
-  const int rem = blockIdx.x - e * per_e;
+  const int slot = blockIdx.x / per_e;
+  const int rem = blockIdx.x - slot * per_e;
   const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
   const int m0 = mt * TM, n0 = nt * TN;
   const bool dense = g.counts == nullptr;
-  const int off = dense ? 0 : g.offsets[e];
-  const int cnt = dense ? g.dense_rows : g.counts[e];
-  const int wm = wave & 1, wn = wave >> 1;  // the wave's 64 x 64 quarter of the tile
+  // Grouped: the experts are taken in descending order of their row counts (ties: lower index
+  // first), so that the longest chains of chunks start first and the short ones fill the end of the
+  // launch.  Every block finds the expert of its rank itself: E <= 256 counts, one comparison loop.
+  // One group: the rows are cut into segments of seg_rows, one slot each, whose partial sums go to
+  // `partial` [segments, M, N] in f32 for wgrad_reduce_kernel to add in order.
+  int e = 0, off, cnt;
+  if (dense) {
+    off = slot * seg_rows;
+    cnt = g.dense_rows - off < seg_rows ? g.dense_rows - off : seg_rows;
+  } else {
+    __shared__ int s_expert, s_cnt[FS2MOE_MAX_EXPERTS];
+    const int mine = tid < g.E ? g.counts[tid] : 0;
+    if (tid < g.E) s_cnt[tid] = mine;
+    __syncthreads();
+    if (tid < g.E) {
+      int rank = 0;
+      for (int j = 0; j < g.E; ++j) {
+        const int cj = s_cnt[j];
+        rank += (cj > mine || (cj == mine && j < tid)) ? 1 : 0;
+      }
+      if (rank == slot) s_expert = tid;
+    }
+    __syncthreads();
+    e = s_expert;
+    off = g.offsets[e];
+    cnt = s_cnt[e];
+  }
+  const int wm = wave & 1, wn = wave >> 1;  // the wave's 128 (m) x 64 (n) part of the tile
   const int lr = lane & 31, lk = lane >> 5;
 
-  f32x16 acc[2][2];  // [tn][tm]
+  f32x16 acc[2][4];  // [tn][tm]
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int b = 0; b < 4; ++b)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
+  // Loads are unconditional, from clamped addresses (a select behind a load would make the wave wait
+  // for it at once); what lies past the expert's rows or the matrix's columns is zeroed when the
+  // registers go to LDS.
   u32x4 ra[PER_THREAD], rb[PER_THREAD];
+  bool va[PER_THREAD], vb[PER_THREAD];
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   auto load_chunk = [&](int r0) {
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
-      const int c = tid + 256 * i;
+      const int c = tid + WAVES * 64 * i;
       const int k = c / ROW_CHUNKS, ch = c % ROW_CHUNKS;
       const int r = r0 + k;
-      ra[i] = zero4;
-      rb[i] = zero4;
-      if (r < cnt) {
-        const int arow = a_map != nullptr ? a_map[off + r] : off + r;
-        if (m0 + ch * VEC < M)
-          ra[i] = *reinterpret_cast<const u32x4*>(A + (size_t)arow * lda + m0 + ch * VEC);
-        if (n0 + ch * VEC < N)
-          rb[i] = *reinterpret_cast<const u32x4*>(B + (size_t)(off + r) * ldb + n0 + ch * VEC);
-      }
+      const bool row_ok = r < cnt;
+      const int rr = off + (row_ok ? r : cnt - 1);  // cnt > 0 here
+      const int arow = a_map != nullptr ? a_map[rr] : rr;
+      const bool a_ok = m0 + ch * VEC < M, b_ok = n0 + ch * VEC < N;
+      va[i] = row_ok && a_ok;
+      vb[i] = row_ok && b_ok;
+      ra[i] = *reinterpret_cast<const u32x4*>(A + (size_t)arow * lda + (a_ok ? m0 + ch * VEC : 0));
+      rb[i] = *reinterpret_cast<const u32x4*>(B + (size_t)rr * ldb + (b_ok ? n0 + ch * VEC : 0));
     }
   };
-  auto store_chunk = [&]() {
+  auto store_chunk = [&](int buf) {
+    uint8_t* sA = smem + buf * 2 * OPB;
+    uint8_t* sB = sA + OPB;
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
-      const int c = tid + 256 * i;
+      const int c = tid + WAVES * 64 * i;
       const int k = c / ROW_CHUNKS, ch = c % ROW_CHUNKS;
       // bf16: chunk ch of row k sits in slot ch ^ ((k & 3) << 2), so that the four consecutive rows
       // a transposing read touches lie 64 bytes apart
       const int slot = BF16 ? (ch ^ ((k & 3) << 2)) : ch;
-      *reinterpret_cast<u32x4*>(sA + k * ROWB + slot * 16) = ra[i];
-      *reinterpret_cast<u32x4*>(sB + k * ROWB + slot * 16) = rb[i];
+      *reinterpret_cast<u32x4*>(sA + k * ROWB + slot * 16) = va[i] ? ra[i] : zero4;
+      *reinterpret_cast<u32x4*>(sB + k * ROWB + slot * 16) = vb[i] ? rb[i] : zero4;
     }
   };
 
@@ -97,63 +134,83 @@ __global__ __launch_bounds__(256) void grouped_wgrad_kernel(
     const int col = cbase + half * 16 + (s & 3) * 4;
     return k * ROWB + (((col >> 3) ^ ((k & 3) << 2)) * 16) + (col & 7) * 2;
   };
-  int fa[2], fb[2];
+  int fa[4], fb[2];
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    fa[t] = BF16 ? tr_addr(wm * 64 + t * 32) : (wm * 64 + t * 32 + lr) * 4;
+  for (int t = 0; t < 4; ++t)
+    fa[t] = BF16 ? tr_addr(wm * 128 + t * 32) : (wm * 128 + t * 32 + lr) * 4;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
     fb[t] = BF16 ? tr_addr(wn * 64 + t * 32) : (wn * 64 + t * 32 + lr) * 4;
-  }
 
-  if (cnt > 0) load_chunk(0);
-  for (int r0 = 0; r0 < cnt; r0 += RK) {
-    __syncthreads();  // the last chunk has been read
-    store_chunk();
-    __syncthreads();
-    if (r0 + RK < cnt) load_chunk(r0 + RK);
+  auto compute_chunk = [&](int buf) {
+    const uint8_t* sA = smem + buf * 2 * OPB;
+    const uint8_t* sB = sA + OPB;
     if constexpr (BF16) {
 #pragma unroll
       for (int ks = 0; ks < RK / 16; ++ks) {
-        bf16x8 af[2], bfr[2];
+        bf16x8 af[4], bfr[2];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < 4; ++t) {
           const uint8_t* pa = sA + fa[t] + ks * 16 * ROWB;
-          const uint8_t* pb = sB + fb[t] + ks * 16 * ROWB;
           af[t] = lds_read_frag_tr(reinterpret_cast<const uint16_t*>(pa),
                                    reinterpret_cast<const uint16_t*>(pa + 4 * ROWB));
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const uint8_t* pb = sB + fb[t] + ks * 16 * ROWB;
           bfr[t] = lds_read_frag_tr(reinterpret_cast<const uint16_t*>(pb),
                                     reinterpret_cast<const uint16_t*>(pb + 4 * ROWB));
         }
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
-          for (int tm = 0; tm < 2; ++tm)
+          for (int tm = 0; tm < 4; ++tm)
             acc[tn][tm] =
                 __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[tn], af[tm], acc[tn][tm], 0, 0, 0);
       }
     } else {
-#pragma unroll 4
+#pragma unroll 2
       for (int ks = 0; ks < RK / 2; ++ks) {
-        float af[2], bfr[2];
+        float af[4], bfr[2];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < 4; ++t)
           af[t] = *reinterpret_cast<const float*>(sA + (2 * ks + lk) * ROWB + fa[t]);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
           bfr[t] = *reinterpret_cast<const float*>(sB + (2 * ks + lk) * ROWB + fb[t]);
-        }
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
-          for (int tm = 0; tm < 2; ++tm)
+          for (int tm = 0; tm < 4; ++tm)
             acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x2f32(bfr[tn], af[tm], acc[tn][tm], 0, 0, 0);
       }
     }
+  };
+
+  // chunk i is multiplied from LDS buffer i & 1 while chunk i + 1 goes from the registers into the
+  // other buffer (read last during chunk i - 1: the barrier that ended it has passed) and chunk i + 2
+  // is loaded
+  const int chunks = (cnt + RK - 1) / RK;
+  if (chunks > 0) {
+    load_chunk(0);
+    store_chunk(0);
+    if (chunks > 1) load_chunk(RK);
+    __syncthreads();
+  }
+  for (int i = 0; i < chunks; ++i) {
+    if (i + 1 < chunks) store_chunk((i + 1) & 1);
+    if (i + 2 < chunks) load_chunk((i + 2) * RK);
+    compute_chunk(i & 1);
+    __syncthreads();
   }
 
   // Accumulator layout: the lane holds row m = lr of fragment tm and columns 8 q + 4 lk + {0..3} of
   // fragment tn in registers 4 q .. 4 q + 3.
   T* Ce = C + (size_t)e * M * N;
+  float* Pe = partial != nullptr ? partial + (size_t)slot * M * N : nullptr;
 #pragma unroll
-  for (int tm = 0; tm < 2; ++tm) {
-    const int m = m0 + wm * 64 + tm * 32 + lr;
+  for (int tm = 0; tm < 4; ++tm) {
+    const int m = m0 + wm * 128 + tm * 32 + lr;
     if (m >= M) continue;
 #pragma unroll
     for (int tn = 0; tn < 2; ++tn) {
@@ -163,7 +220,10 @@ __global__ __launch_bounds__(256) void grouped_wgrad_kernel(
         if (n >= N) continue;  // N is a multiple of 4: the four columns are in or out together
         const float v0 = acc[tn][tm][4 * q], v1 = acc[tn][tm][4 * q + 1];
         const float v2 = acc[tn][tm][4 * q + 2], v3 = acc[tn][tm][4 * q + 3];
-        if constexpr (BF16) {
+        if (Pe != nullptr) {
+          f32x4 o = {v0, v1, v2, v3};
+          *reinterpret_cast<f32x4*>(Pe + (size_t)m * N + n) = o;
+        } else if constexpr (BF16) {
           u32x2 o = {pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
           *reinterpret_cast<u32x2*>(Ce + (size_t)m * N + n) = o;
         } else {
@@ -172,6 +232,23 @@ __global__ __launch_bounds__(256) void grouped_wgrad_kernel(
         }
       }
     }
+  }
+}
+
+// out[i] = sum over the segments, in order, of partial[s][i]; one rounding.
+template <typename T>
+__global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ partial,
+                                                           int segments, int64_t n,
+                                                           T* __restrict__ out) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= n) return;  // n is a multiple of 4
+  f32x4 acc = *reinterpret_cast<const f32x4*>(partial + i);
+  for (int s = 1; s < segments; ++s) acc += *reinterpret_cast<const f32x4*>(partial + (size_t)s * n + i);
+  if constexpr (sizeof(T) == 2) {
+    u32x2 o = {pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3])};
+    *reinterpret_cast<u32x2*>(out + i) = o;
+  } else {
+    *reinterpret_cast<f32x4*>(out + i) = acc;
   }
 }
 
@@ -239,10 +316,37 @@ __global__ __launch_bounds__(256) void pair_dot_kernel(const T* __restrict__ a,
   const int lane = threadIdx.x & 63;
   const size_t ar = (size_t)a_rows[p] * D, br = (size_t)(p / K) * D;
   float s = 0.f;
-  for (int d = lane; d < D; d += 64) {
-    float av = Elem<T>::load(a + ar + d);
-    if (a2 != nullptr) av += Elem<T>::load(a2 + ar + d);
-    s += av * Elem<T>::load(b + br + d);
+  constexpr int VEC = 16 / sizeof(T);
+  if (D % VEC == 0) {
+    // 16 bytes per lane and load
+    for (int d = lane * VEC; d < D; d += 64 * VEC) {
+      const u32x4 av = *reinterpret_cast<const u32x4*>(a + ar + d);
+      const u32x4 bv = *reinterpret_cast<const u32x4*>(b + br + d);
+      u32x4 cv = {0u, 0u, 0u, 0u};
+      if (a2 != nullptr) cv = *reinterpret_cast<const u32x4*>(a2 + ar + d);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if constexpr (sizeof(T) == 2) {
+          float x0 = __uint_as_float(av[j] << 16), x1 = __uint_as_float(av[j] & 0xffff0000u);
+          if (a2 != nullptr) {
+            x0 += __uint_as_float(cv[j] << 16);
+            x1 += __uint_as_float(cv[j] & 0xffff0000u);
+          }
+          s += x0 * __uint_as_float(bv[j] << 16);
+          s += x1 * __uint_as_float(bv[j] & 0xffff0000u);
+        } else {
+          float x0 = __uint_as_float(av[j]);
+          if (a2 != nullptr) x0 += __uint_as_float(cv[j]);
+          s += x0 * __uint_as_float(bv[j]);
+        }
+      }
+    }
+  } else {
+    for (int d = lane; d < D; d += 64) {
+      float av = Elem<T>::load(a + ar + d);
+      if (a2 != nullptr) av += Elem<T>::load(a2 + ar + d);
+      s += av * Elem<T>::load(b + br + d);
+    }
   }
   s = wave_sum_f32(s);
   if (lane == 0) out[p] = s;
@@ -313,10 +417,28 @@ __global__ __launch_bounds__(256) void router_backward_kernel(
 
 using namespace fs2moe;
 
+// One group with fewer tiles than the chip has CUs: the rows are cut into this many segments.
+static int wgrad_segments(int64_t rows, int M, int N) {
+  const int64_t tiles = (int64_t)((M + wgk::TM - 1) / wgk::TM) * ((N + wgk::TN - 1) / wgk::TN);
+  if (tiles >= 128) return 1;
+  int64_t s = 256 / tiles;
+  const int64_t most = rows / 256;  // at least 256 rows per segment
+  s = s < most ? s : most;
+  return s >= 2 ? (int)s : 1;
+}
+
+extern "C" int64_t fs2moe_grouped_wgrad_workspace_bytes(int32_t grouped, int32_t M, int32_t N,
+                                                        int64_t max_rows) {
+  if (M < 1 || N < 1 || max_rows < 0) return -1;
+  if (grouped) return 0;
+  const int s = wgrad_segments(max_rows, M, N);
+  return s > 1 ? (int64_t)s * M * N * 4 : 0;
+}
+
 extern "C" int fs2moe_grouped_wgrad(const void* a, const int32_t* a_row_map, const void* b,
                                     const int32_t* counts, const int32_t* offsets, int32_t E,
                                     int32_t M, int32_t N, int64_t max_rows, int32_t dtype, void* dw,
-                                    void* stream) {
+                                    void* workspace, int64_t workspace_bytes, void* stream) {
   FS2_REQUIRE(a && b && dw, "grouped_wgrad: null pointer");
   FS2_REQUIRE((counts == nullptr) == (offsets == nullptr), "grouped_wgrad: counts without offsets");
   FS2_REQUIRE(E >= 1 && E <= FS2MOE_MAX_EXPERTS && (counts != nullptr || E == 1),
@@ -327,23 +449,59 @@ extern "C" int fs2moe_grouped_wgrad(const void* a, const int32_t* a_row_map, con
               "grouped_wgrad: M=%d and N=%d must be positive multiples of %d", M, N, vec);
   FS2_REQUIRE(max_rows >= 0 && max_rows < (1ll << 31), "grouped_wgrad: max_rows=%lld",
               (long long)max_rows);
-  FS2_REQUIRE(aligned16(a) && aligned16(b) && aligned16(dw),
+  FS2_REQUIRE(aligned16(a) && aligned16(b) && aligned16(dw) && aligned16(workspace),
               "grouped_wgrad: buffers must be 16-byte aligned");
   const int m_tiles = (M + wgk::TM - 1) / wgk::TM, n_tiles = (N + wgk::TN - 1) / wgk::TN;
-  const int64_t blocks = (int64_t)E * m_tiles * n_tiles;
+  // one group: segments of its rows (each a slot of the grid) when there is scratch for their sums
+  int segments = 1;
+  if (counts == nullptr) {
+    segments = wgrad_segments(max_rows, M, N);
+    if (workspace == nullptr || workspace_bytes < (int64_t)segments * M * N * 4) segments = 1;
+  }
+  const int slots = counts != nullptr ? E : segments;
+  const int seg_rows = (int)(((max_rows + segments - 1) / segments + 15) / 16 * 16);
+  float* partial = segments > 1 ? static_cast<float*>(workspace) : nullptr;
+  const int64_t blocks = (int64_t)slots * m_tiles * n_tiles;
   FS2_REQUIRE(blocks <= 0x7fffffffll, "grouped_wgrad: too many tiles");
   Groups g{counts, offsets, E, (int)max_rows};
   hipStream_t st = static_cast<hipStream_t>(stream);
+  auto kb = grouped_wgrad_kernel<uint16_t>;
+  auto kf = grouped_wgrad_kernel<float>;
+  static bool attr_set = false;  // benign race: setting the attribute is idempotent
+  if (!attr_set) {
+    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(kb),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, wgk::SMEM_BYTES);
+    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(kf),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, wgk::SMEM_BYTES);
+    if (e1 != hipSuccess || e2 != hipSuccess) {
+      set_error("grouped_wgrad: cannot reserve %d bytes of LDS: %s", wgk::SMEM_BYTES,
+                hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+      return FS2MOE_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
   if (dtype == FS2MOE_BF16)
-    hipLaunchKernelGGL(grouped_wgrad_kernel<uint16_t>, dim3((unsigned)blocks), dim3(256), 0, st,
+    hipLaunchKernelGGL(kb, dim3((unsigned)blocks), dim3(wgk::WAVES * 64), wgk::SMEM_BYTES, st,
                        static_cast<const uint16_t*>(a), a_row_map, M,
                        static_cast<const uint16_t*>(b), N, static_cast<uint16_t*>(dw), M, N, g,
-                       m_tiles, n_tiles);
+                       m_tiles, n_tiles, seg_rows, partial);
   else
-    hipLaunchKernelGGL(grouped_wgrad_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, st,
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(wgk::WAVES * 64), wgk::SMEM_BYTES, st,
                        static_cast<const float*>(a), a_row_map, M, static_cast<const float*>(b), N,
-                       static_cast<float*>(dw), M, N, g, m_tiles, n_tiles);
-  return check_launch("grouped_wgrad");
+                       static_cast<float*>(dw), M, N, g, m_tiles, n_tiles, seg_rows, partial);
+  if (int rc = check_launch("grouped_wgrad")) return rc;
+  if (segments > 1) {
+    const int64_t n = (int64_t)M * N;
+    const unsigned rblocks = (unsigned)((n / 4 + 255) / 256);
+    if (dtype == FS2MOE_BF16)
+      hipLaunchKernelGGL(wgrad_reduce_kernel<uint16_t>, dim3(rblocks), dim3(256), 0, st, partial,
+                         segments, n, static_cast<uint16_t*>(dw));
+    else
+      hipLaunchKernelGGL(wgrad_reduce_kernel<float>, dim3(rblocks), dim3(256), 0, st, partial,
+                         segments, n, static_cast<float*>(dw));
+    return check_launch("wgrad_reduce");
+  }
+  return FS2MOE_OK;
 }
 
 extern "C" int fs2moe_swiglu_backward(const void* g, const void* u, const void* dh, int64_t rows,

@@ -287,10 +287,17 @@ int fs2moe_grouped_gemm(const void* a, const int32_t* row_map, const int32_t* co
  * (A = the experts' input rows or h, B = the gradient of the product) and of ffn.py:374-395.
  *   a [rows, M] dtype (row r read from a[a_row_map[r]] when a_row_map is given)   b [rows, N] dtype
  *   dw [E*M, N] dtype (out).  M and N multiples of 8 (bf16) or 4 (f32).
+ *   workspace: optional device scratch of fs2moe_grouped_wgrad_workspace_bytes(grouped, ...) bytes,
+ *   16-byte aligned (grouped = 0 when counts is NULL).  One group with few output tiles (the router's
+ *   gradient) then has its rows cut into segments whose f32 partial sums a second kernel adds in
+ *   order; without it (NULL, or fewer bytes) each tile walks all rows.
  */
+int64_t fs2moe_grouped_wgrad_workspace_bytes(int32_t grouped, int32_t M, int32_t N,
+                                             int64_t max_rows);
 int fs2moe_grouped_wgrad(const void* a, const int32_t* a_row_map, const void* b,
                          const int32_t* counts, const int32_t* offsets, int32_t E, int32_t M,
-                         int32_t N, int64_t max_rows, int32_t dtype, void* dw, void* stream);
+                         int32_t N, int64_t max_rows, int32_t dtype, void* dw, void* workspace,
+                         int64_t workspace_bytes, void* stream);
 
 /*
  * SwiGLU backward, element-wise: h = SiLU(g) * u, dg = dh * u * SiLU'(g), du = dh * SiLU(g).
