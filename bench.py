@@ -29,8 +29,13 @@ MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3, "fp8": 5000.0}  # dense, publ
 # HBM bytes per launch of the dominant kernel pair, from `rocprofv3 --pmc FETCH_SIZE` and
 # `--pmc WRITE_SIZE` runs of this script (see profiles/); None until measured for a workload.
 MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
-    # profiles/bench_qwen3_30b_a3b_all_kernels.md: gate/up 1395 + 101 MB, down 690 + 270 MB
-    "qwen3_30b_a3b": 2.456e9,
+    # profiles/bench_<workload>_all_kernels.md, the two launches of fs2moe_grouped_swiglu together
+    # (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0 against a 256 MiB copy)
+    "qwen3_30b_a3b": 2.649e9,     # gate/up 1548 + 101 MB, down 729 + 270 MB
+    "mixtral_8x7b": 15.091e9,     # gate/up 10404 + 470 MB, down 4081 + 136 MB
+    "llama4_scout": 6.632e9,      # routed experts only: gate/up 4234 + 134 MB, down 2178 + 86 MB
+    "small_fp32": 0.862e9,        # gate/up 398 + 46 MB, down 401 + 17 MB
+    "qwen3_decode_fp8": 0.224e9,  # gate/up 142 + 1 MB, down 77 + 4 MB
 }
 
 
@@ -50,6 +55,9 @@ def parse_args():
     p.add_argument("--stage-reps", type=int, default=20)
     p.add_argument("--graph", action="store_true",
                    help="time replays of one captured HIP graph of the layer instead of eager calls")
+    p.add_argument("--training-step", action="store_true",
+                   help="also time forward + backward of the module (reported beside the metric, "
+                        "not part of it; bf16 / fp32 weights only)")
     p.add_argument("--calibration-copy", action="store_true",
                    help="also run a 256 MiB device copy (reference point for rocprofv3 byte counters)")
     return p.parse_args()
@@ -176,6 +184,38 @@ def cpu_baseline(wl, seconds: float) -> dict:
         "kind": "port",
         "sample": f"dense reference formulation in {str(dt).replace('torch.', '')} on the first {n} of "
                   f"{spec.num_tokens} tokens, one timed pass of {dt_s:.2f} s (after shorter passes that sized it)",
+    }
+
+
+def training_step(module, x3, steps: int) -> dict:
+    """Forward + backward of the module with every parameter and the input requiring a gradient
+    (the library's backward kernels): milliseconds per step and the peak memory torch saw."""
+    import torch
+
+    module.train().requires_grad_(True)
+    x = x3.detach().clone().requires_grad_(True)
+    grad = torch.randn_like(x)
+
+    def step():
+        for p in module.parameters():
+            p.grad = None
+        x.grad = None
+        module(x).backward(grad)
+
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    module.requires_grad_(False).eval()
+    return {
+        "ms": round(ms, 4), "steps": steps,
+        "peak_memory_gib": round(torch.cuda.max_memory_allocated() / 2**30, 2),
+        "what": "forward + backward of the module (gradients of the input and of every parameter)",
     }
 
 
@@ -346,6 +386,8 @@ def main() -> int:
             "what": "x + layer(rms_norm(x)) in one call: norm in the router kernel, residual in combine",
         },
     }
+    if args.training_step and spec.weight_dtype != "fp8":
+        result["training_step"] = training_step(module, x3, max(3, args.steps // 10))
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(wl, args.cpu_seconds)
     print(json.dumps(result), flush=True)
