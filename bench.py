@@ -177,13 +177,22 @@ def cpu_baseline(wl, seconds: float) -> dict:
         want = int(n * min(16.0, 0.9 * seconds / max(dt_s, 1e-9)))
         n = min(spec.num_tokens, max(n + 64, want // 64 * 64))
         dt_s = run(n)
+    # the whole workload in less than the target time: repeat the pass and report the mean
+    passes = 1
+    if dt_s < 0.6 * seconds:
+        passes = int(min(10, max(2, 0.9 * seconds / max(dt_s, 1e-9))))
+        t0 = time.perf_counter()
+        for _ in range(passes):
+            run(n)
+        dt_s = (time.perf_counter() - t0) / passes
     return {
         "value": n / dt_s,
         "unit": "tokens/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
         "sample": f"dense reference formulation in {str(dt).replace('torch.', '')} on the first {n} of "
-                  f"{spec.num_tokens} tokens, one timed pass of {dt_s:.2f} s (after shorter passes that sized it)",
+                  f"{spec.num_tokens} tokens, mean of {passes} timed pass(es) of {dt_s:.2f} s each "
+                  f"(after shorter passes that sized the sample)",
     }
 
 
