@@ -58,6 +58,10 @@ def parse_args():
     p.add_argument("--training-step", action="store_true",
                    help="also time forward + backward of the module (reported beside the metric, "
                         "not part of it; bf16 / fp32 weights only)")
+    p.add_argument("--vendor-gemm", action="store_true",
+                   help="also time the expert GEMM shapes as three dense products in the vendor's "
+                        "library (torch.matmul -> hipBLASLt): a yardstick for what the matrix pipes "
+                        "sustain on this data, reported beside the metric")
     p.add_argument("--calibration-copy", action="store_true",
                    help="also run a 256 MiB device copy (reference point for rocprofv3 byte counters)")
     return p.parse_args()
@@ -193,6 +197,46 @@ def cpu_baseline(wl, seconds: float) -> dict:
         "sample": f"dense reference formulation in {str(dt).replace('torch.', '')} on the first {n} of "
                   f"{spec.num_tokens} tokens, mean of {passes} timed pass(es) of {dt_s:.2f} s each "
                   f"(after shorter passes that sized the sample)",
+    }
+
+
+def vendor_gemm(spec, dev) -> dict:
+    """The routed rows as ONE group through the vendor's dense bf16 GEMM: (T K, D) x (D, F) twice and
+    (T K, F) x (F, D), on data drawn like the workload's.  No grouping, no skew, no gather, no gate:
+    what the same flops cost in the library AMD ships, on this box, on this kind of data."""
+    import torch
+
+    rows, d, f = spec.num_tokens * spec.top_k, spec.model_dim, spec.inner_dim
+    g = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn(rows, d, device=dev, generator=g).to(torch.bfloat16)
+    h = torch.randn(rows, f, device=dev, generator=g).to(torch.bfloat16)
+    w1 = (0.02 * torch.randn(d, f, device=dev, generator=g)).to(torch.bfloat16)
+    w2 = (0.02 * torch.randn(f, d, device=dev, generator=g)).to(torch.bfloat16)
+
+    def timed(fn, reps=20):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        best = float("inf")
+        for _ in range(3):
+            a.record()
+            for _ in range(reps):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            best = min(best, a.elapsed_time(b) / reps)
+        return best
+
+    with torch.no_grad():
+        up_ms = timed(lambda: torch.matmul(x, w1))
+        down_ms = timed(lambda: torch.matmul(h, w2))
+    total = 2 * up_ms + down_ms
+    flops = 6.0 * rows * d * f
+    return {
+        "ms": round(total, 4), "gate_or_up_ms": round(up_ms, 4), "down_ms": round(down_ms, 4),
+        "achieved_tflops": round(flops / (total * 1e-3) / 1e12, 1),
+        "what": "torch.matmul (hipBLASLt) on the routed rows as one dense group: gate, up and down products",
     }
 
 
@@ -395,6 +439,8 @@ def main() -> int:
             "what": "x + layer(rms_norm(x)) in one call: norm in the router kernel, residual in combine",
         },
     }
+    if args.vendor_gemm and spec.dtype == "bf16":
+        result["vendor_gemm"] = vendor_gemm(spec, dev)
     if args.training_step and spec.weight_dtype != "fp8":
         result["training_step"] = training_step(module, x3, max(3, args.steps // 10))
     if not args.no_cpu_baseline:
