@@ -13,6 +13,23 @@ namespace fs2moe {
 constexpr int kDispTok = 256;  // tokens per block in the counting pass (= threads per block)
 constexpr int kDispWords = kDispTok / 32;
 
+// The experts of token t, -1 where there is none (t past T, k past K, an index outside [0, E)).
+// Every load is issued, from an address inside the array, before any result is looked at: a load
+// behind a condition is waited for on the spot, one round trip per k.
+__device__ __forceinline__ void load_token_experts(const int32_t* __restrict__ topk_idx, int t,
+                                                   int T, int K, int E,
+                                                   int (&ek)[FS2MOE_MAX_TOP_K]) {
+  const bool has_token = t < T;
+  const int32_t* mine = topk_idx + (has_token ? (size_t)t * K : 0);
+#pragma unroll
+  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) ek[k] = mine[k < K ? k : 0];
+#pragma unroll
+  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) {
+    const int e = ek[k];
+    ek[k] = (has_token && k < K && e >= 0 && e < E) ? e : -1;
+  }
+}
+
 __global__ __launch_bounds__(kDispTok) void dispatch_count_kernel(
     const int32_t* __restrict__ topk_idx, int T, int K, int E, int32_t* __restrict__ block_counts,
     int32_t* __restrict__ rank) {
@@ -27,13 +44,10 @@ __global__ __launch_bounds__(kDispTok) void dispatch_count_kernel(
   const uint32_t bit = 1u << (tid & 31);
   // the token's experts stay in registers between the two passes
   int ek[FS2MOE_MAX_TOP_K];
+  load_token_experts(topk_idx, t, T, K, E, ek);
 #pragma unroll
-  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) {
-    int e = -1;
-    if (k < K && t < T) e = topk_idx[(size_t)t * K + k];
-    ek[k] = (e >= 0 && e < E) ? e : -1;
+  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k)
     if (ek[k] >= 0) atomicOr(&s_bits[ek[k] * kDispWords + word], bit);
-  }
   __syncthreads();
   for (int i = tid; i < E * kDispWords; i += kDispTok) {
     const int e = i / kDispWords, w = i % kDispWords;
@@ -226,13 +240,10 @@ __global__ __launch_bounds__(kDispTok) void dispatch_small_kernel(
   const int word = tid >> 5;
   const uint32_t bit = 1u << (tid & 31);
   int ek[FS2MOE_MAX_TOP_K];
+  load_token_experts(topk_idx, t, T, K, E, ek);
 #pragma unroll
-  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) {
-    int e = -1;
-    if (k < K && t < T) e = topk_idx[(size_t)t * K + k];
-    ek[k] = (e >= 0 && e < E) ? e : -1;
+  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k)
     if (ek[k] >= 0) atomicOr(&s_bits[ek[k] * kDispWords + word], bit);
-  }
   __syncthreads();
   for (int i = tid; i < E * kDispWords; i += kDispTok) {
     const int e = i / kDispWords, w = i % kDispWords;
