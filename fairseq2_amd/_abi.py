@@ -15,7 +15,7 @@ from torch import Tensor
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfs2moe.so")
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
@@ -55,6 +55,11 @@ _PROTOTYPES = {
          c_void_p],
     ),
     "fs2moe_grouped_swiglu_fuses_gather": (c_int32, [c_int32, c_int32, c_int32, c_int32]),
+    "fs2moe_grouped_swiglu_keeps": (c_int32, [c_int32, c_int32, c_int64, c_int32]),
+    "fs2moe_grouped_swiglu_keep": (
+        c_int32,
+        [c_void_p] * 7 + [c_int32] * 3 + [c_int64, c_int32] + [c_void_p] * 5,
+    ),
     "fs2moe_dense_swiglu": (
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p,
@@ -397,6 +402,44 @@ def grouped_swiglu(
     return ye, h
 
 
+def keeps_products(model_dim: int, inner_dim: int, rows: int, act_dtype: torch.dtype) -> bool:
+    """Whether :func:`grouped_swiglu_keep` exists for these sizes and this type."""
+    return bool(load().fs2moe_grouped_swiglu_keeps(model_dim, inner_dim, rows, dtype_code(act_dtype)))
+
+
+def grouped_swiglu_keep(
+    xe: Tensor,
+    counts: Tensor,
+    offsets: Tensor,
+    w_gate: Tensor,
+    w_up: Tensor,
+    w_down: Tensor,
+    num_experts: int,
+    row_map: Tensor | None = None,
+) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """:func:`grouped_swiglu` that also returns the gate and the up product: ``(ye, h, g, u)``."""
+    lib = load()
+    rows, d = xe.shape
+    if row_map is not None:
+        rows = row_map.shape[0]
+    f = w_down.shape[0] // num_experts
+    if w_gate.shape != (num_experts * d, f) or w_up.shape != w_gate.shape:
+        raise ValueError("gate/up weights must be (E*D, F)")
+    if w_down.shape != (num_experts * f, d):
+        raise ValueError("down weights must be (E*F, D)")
+    for name, w in (("w_gate", w_gate), ("w_up", w_up), ("w_down", w_down)):
+        _same(name, w, w.shape, xe.dtype, xe.device)
+    g, u, h = (torch.empty((rows, f), dtype=xe.dtype, device=xe.device) for _ in range(3))
+    ye = torch.empty((rows, d), dtype=xe.dtype, device=xe.device)
+    rc = lib.fs2moe_grouped_swiglu_keep(
+        _ptr(xe), _ptr(row_map), _ptr(counts), _ptr(offsets), _ptr(w_gate), _ptr(w_up),
+        _ptr(w_down), num_experts, d, f, rows, dtype_code(xe.dtype), _ptr(g), _ptr(u), _ptr(h),
+        _ptr(ye), _stream(),
+    )
+    _check(rc, "fs2moe_grouped_swiglu_keep")
+    return ye, h, g, u
+
+
 def fuses_gather(model_dim: int, inner_dim: int, act_dtype: torch.dtype, w_dtype: torch.dtype) -> bool:
     """Whether :func:`grouped_swiglu` takes a ``row_map`` for these sizes and types."""
     return bool(
@@ -554,20 +597,22 @@ def grouped_wgrad(
     return dw
 
 
-def swiglu_backward(g: Tensor, u: Tensor, dh: Tensor) -> tuple[Tensor, Tensor, Tensor]:
-    """``(h, dg, du)`` of ``h = SiLU(g) * u`` given ``dh``; ``dg`` and ``du`` overwrite ``g`` and ``u``."""
+def swiglu_backward(g: Tensor, u: Tensor, dh: Tensor, in_place: bool = True) -> tuple[Tensor, Tensor, Tensor]:
+    """``(h, dg, du)`` of ``h = SiLU(g) * u`` given ``dh``; ``dg`` and ``du`` overwrite ``g`` and
+    ``u`` unless ``in_place`` is false."""
     lib = load()
     _same("u", u, g.shape, g.dtype, g.device)
     _same("dh", dh, g.shape, g.dtype, g.device)
     if not g.is_contiguous():
         raise ValueError("g must be contiguous")
     h = torch.empty_like(g)
+    dg, du = (g, u) if in_place else (torch.empty_like(g), torch.empty_like(u))
     rc = lib.fs2moe_swiglu_backward(
-        _ptr(g), _ptr(u), _ptr(dh), g.shape[0], g.shape[1], dtype_code(g.dtype), _ptr(h), _ptr(g),
-        _ptr(u), _stream(),
+        _ptr(g), _ptr(u), _ptr(dh), g.shape[0], g.shape[1], dtype_code(g.dtype), _ptr(h), _ptr(dg),
+        _ptr(du), _stream(),
     )
     _check(rc, "fs2moe_swiglu_backward")
-    return h, g, u
+    return h, dg, du
 
 
 def pair_dot(a: Tensor, a_rows: Tensor, b: Tensor, a2: Tensor | None = None) -> Tensor:

@@ -10,7 +10,8 @@ derivation is written out once, against ``moe.py:102-157``, ``experts.py:102-112
                                                                          or s_k = 1, c_k = w_k
     dye      = c * dout[token]                 gathered into expert order      -> fs2moe_dispatch
     dh       = dye @ Wd^T                                                      -> fs2moe_grouped_gemm
-    g, u     = xe @ Wg, xe @ Wu                recomputed, not stored          -> fs2moe_grouped_gemm
+    g, u     = xe @ Wg, xe @ Wu                kept by the forward pass        -> fs2moe_grouped_swiglu_keep
+                                                or computed again               -> fs2moe_grouped_gemm
     dg, du   = SwiGLU'(g, u, dh),  h = SiLU(g) u                               -> fs2moe_swiglu_backward
     dWd, dWg, dWu = h^T dye, xe^T dg, xe^T du  per expert                      -> fs2moe_grouped_wgrad
     dxe      = dg @ Wg^T + du @ Wu^T                                           -> fs2moe_grouped_gemm
@@ -37,16 +38,22 @@ def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg):
     score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
     idx, w, logits = _abi.router_topk(x, router, cfg["router_bias"], k, score_fn, renorm, want_logits=True)
     disp = _abi.dispatch(idx, w, x, e, tile_m, scale_input, gather=True)
-    ye, _ = _abi.grouped_swiglu(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
+    # where the expert kernel can, it leaves the gate and the up product behind for the backward
+    # pass (what autograd would save); otherwise backward_from computes them again
+    g = u = None
+    if _abi.keeps_products(x.shape[1], wd.shape[0] // e, disp.xe.shape[0], x.dtype):
+        ye, _, g, u = _abi.grouped_swiglu_keep(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
+    else:
+        ye, _ = _abi.grouped_swiglu(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
     base = _abi.dense_swiglu(x, sg, su, sd) if sg is not None else None
     out = _abi.combine(ye, disp.inv_perm, idx, w, base, not scale_input, out=base, residual=residual)
-    return out, (idx, w, logits, disp.counts, disp.offsets, disp.inv_perm, disp.xe, ye)
+    return out, (idx, w, logits, disp.counts, disp.offsets, disp.inv_perm, disp.xe, ye, g, u)
 
 
 def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
     """Gradients ``(dx, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd)`` (None where ``need`` -- in
     that order -- says so) from the output gradient and the intermediates of :func:`forward_saving`."""
-    idx, w, logits, counts, offsets, inv_perm, xe, ye = saved
+    idx, w, logits, counts, offsets, inv_perm, xe, ye, g, u = saved
     e, tile_m = cfg["num_experts"], cfg["tile_m"]
     score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
     dout = dout.contiguous()
@@ -57,9 +64,12 @@ def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
     # the permutation is the forward pass's: dispatch is deterministic
     dye = _abi.dispatch(idx, w, dout, e, tile_m, not scale_input, gather=True).xe
     dh = _abi.grouped_gemm(dye, wd, OUT_IN, **grp)
-    g = _abi.grouped_gemm(xe, wg, IN_OUT, **grp)
-    u = _abi.grouped_gemm(xe, wu, IN_OUT, **grp)
-    h, dg, du = _abi.swiglu_backward(g, u, dh)
+    if g is None:
+        g = _abi.grouped_gemm(xe, wg, IN_OUT, **grp)
+        u = _abi.grouped_gemm(xe, wu, IN_OUT, **grp)
+        h, dg, du = _abi.swiglu_backward(g, u, dh)  # in place over g and u
+    else:
+        h, dg, du = _abi.swiglu_backward(g, u, dh, in_place=False)  # g, u are autograd's to keep
     d_wd = _abi.grouped_wgrad(h, dye, **grp) if need[4] else None
     d_wg = _abi.grouped_wgrad(xe, dg, **grp) if need[2] else None
     d_wu = _abi.grouped_wgrad(xe, du, **grp) if need[3] else None

@@ -46,10 +46,14 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // Which tile: slots (an expert, by rank as below, or a segment of the one group's rows) in launch
+  // order, and within a slot row block minor: blocks reach the 8 XCDs round-robin (block b runs on
+  // XCD b % 8, each with its own L2), so with 8 row blocks the tiles of a slot that share an XCD
+  // share their block of A's columns.
   const int per_e = m_tiles * n_tiles;
   const int slot = blockIdx.x / per_e;
   const int rem = blockIdx.x - slot * per_e;
-  const int mt = rem / n_tiles, nt = rem - mt * n_tiles;
+  const int nt = rem / m_tiles, mt = rem - nt * m_tiles;
   const int m0 = mt * TM, n0 = nt * TN;
   const bool dense = g.counts == nullptr;
   // Grouped: the experts are taken in descending order of their row counts (ties: lower index
@@ -208,6 +212,44 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
   // fragment tn in registers 4 q .. 4 q + 3.
   T* Ce = C + (size_t)e * M * N;
   float* Pe = partial != nullptr ? partial + (size_t)slot * M * N : nullptr;
+  if constexpr (BF16) {
+    if (Pe == nullptr) {
+      // Through LDS (free after the loop's last barrier), so that a store instruction writes 8 rows
+      // of 128 contiguous bytes instead of 32 rows of 16: the wave puts a 32 (m) x 64 (n) fragment
+      // row into its own 4.25 KB as bf16, rows 136 bytes apart, and reads it back 16 bytes per lane.
+      constexpr int LDE = 136;
+      uint8_t* sw = smem + wave * 8192;
+      const int rrow = lane >> 3, rcol = lane & 7;
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm) {
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            u32x2 o = {pack_bf16x2(acc[tn][tm][4 * q], acc[tn][tm][4 * q + 1]),
+                       pack_bf16x2(acc[tn][tm][4 * q + 2], acc[tn][tm][4 * q + 3])};
+            *reinterpret_cast<u32x2*>(sw + lr * LDE + (tn * 32 + 8 * q + 4 * lk) * 2) = o;
+          }
+        // the wave's own LDS traffic runs in order; the compiler must not move the reads (other
+        // lanes' data) above the writes, nor the next round's writes above these reads
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const int n = n0 + wn * 64 + rcol * 8;
+#pragma unroll
+        for (int p8 = 0; p8 < 4; ++p8) {
+          const int row = p8 * 8 + rrow;
+          const u32x2 lo = *reinterpret_cast<const u32x2*>(sw + row * LDE + rcol * 16);
+          const u32x2 hi = *reinterpret_cast<const u32x2*>(sw + row * LDE + rcol * 16 + 8);
+          const int m = m0 + wm * 128 + tm * 32 + row;
+          if (m < M && n < N) {  // N is a multiple of 8: the eight columns are in or out together
+            u32x4 o = {lo[0], lo[1], hi[0], hi[1]};
+            *reinterpret_cast<u32x4*>(Ce + (size_t)m * N + n) = o;
+          }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int tm = 0; tm < 4; ++tm) {
     const int m = m0 + wm * 128 + tm * 32 + lr;

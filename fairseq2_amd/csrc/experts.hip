@@ -334,21 +334,28 @@ static int launch_dma_pair(const void* x, const int32_t* row_map, const Groups& 
                            int64_t rows_bound, const void* w_gate, const void* w_up,
                            const void* w_down, const float* s_gate, const float* s_up,
                            const float* s_down, int D, int F, void* h, void* y,
-                           hipStream_t stream) {
+                           hipStream_t stream, void* g_keep = nullptr, void* u_keep = nullptr) {
   using namespace dma;
   const int groups = g.counts ? g.E : 0;
+  // the gate/up kernel, or its variant that also stores the two products (plain bf16 weights only)
+  constexpr bool CAN_KEEP = BLAYOUT == FS2MOE_W_IN_OUT;
   auto k1 = glu_gemm_bf16_dma_kernel<true, BLAYOUT>;
+  auto k1k = glu_gemm_bf16_dma_kernel<true, BLAYOUT, CAN_KEEP>;
   auto k2 = glu_gemm_bf16_dma_kernel<false, BLAYOUT>;
+  if (g_keep != nullptr && !CAN_KEEP) {
+    set_error("experts: the products are kept with bf16 weights in the (in, out) layout only");
+    return FS2MOE_ERR_UNSUPPORTED;
+  }
   static bool attr_set = false;  // benign race: setting the attribute is idempotent
   if (!attr_set) {
-    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(k1),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
-    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(k2),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
-    if (e1 != hipSuccess || e2 != hipSuccess) {
-      set_error("experts: cannot reserve %d bytes of LDS: %s", SMEM_BYTES,
-                hipGetErrorString(e1 != hipSuccess ? e1 : e2));
-      return FS2MOE_ERR_LAUNCH;
+    const void* ks[3] = {reinterpret_cast<const void*>(k1), reinterpret_cast<const void*>(k1k),
+                         reinterpret_cast<const void*>(k2)};
+    for (const void* k : ks) {
+      hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+      if (e != hipSuccess) {
+        set_error("experts: cannot reserve %d bytes of LDS: %s", SMEM_BYTES, hipGetErrorString(e));
+        return FS2MOE_ERR_LAUNCH;
+      }
     }
     attr_set = true;
   }
@@ -367,10 +374,13 @@ static int launch_dma_pair(const void* x, const int32_t* row_map, const Groups& 
     }
   }
   const unsigned g1 = (unsigned)num_blocks, g2 = (unsigned)num_blocks;
-  hipLaunchKernelGGL(k1, dim3(g1), dim3(NWAVES * 64), SMEM_BYTES, stream,
+  // (the variant that keeps the products takes their destinations in the two scale arguments)
+  hipLaunchKernelGGL(g_keep != nullptr ? k1k : k1, dim3(g1), dim3(NWAVES * 64), SMEM_BYTES, stream,
                      static_cast<const uint16_t*>(x), row_map, D,
-                     static_cast<const uint16_t*>(w_gate), static_cast<const uint16_t*>(w_up), s_gate,
-                     s_up, static_cast<uint16_t*>(h), F, D, F, g, nt1);
+                     static_cast<const uint16_t*>(w_gate), static_cast<const uint16_t*>(w_up),
+                     g_keep != nullptr ? static_cast<const float*>(g_keep) : s_gate,
+                     g_keep != nullptr ? static_cast<const float*>(u_keep) : s_up,
+                     static_cast<uint16_t*>(h), F, D, F, g, nt1);
   if (int rc = check_launch("glu_gemm_bf16_dma<gate,up>")) return rc;
   hipLaunchKernelGGL(k2, dim3(g2), dim3(NWAVES * 64), SMEM_BYTES, stream,
                      static_cast<const uint16_t*>(h), static_cast<const int32_t*>(nullptr), F,
@@ -446,6 +456,39 @@ extern "C" int fs2moe_grouped_swiglu_fuses_gather(int32_t D, int32_t F, int32_t 
   if (D <= 0 || F <= 0) return 0;
   if (w_dtype == FS2MOE_FP8_E4M3) return (act_dtype == FS2MOE_BF16 && D % 64 == 0 && F % 64 == 0) ? 1 : 0;
   return (w_dtype == act_dtype && dma_path_applies(act_dtype, D, F)) ? 1 : 0;
+}
+
+extern "C" int fs2moe_grouped_swiglu_keeps(int32_t D, int32_t F, int64_t max_rows,
+                                           int32_t act_dtype) {
+  if (D <= 0 || F <= 0 || max_rows < 0) return 0;
+  return (dma_path_applies(act_dtype, D, F) && dma_offsets_fit(max_rows, D, F)) ? 1 : 0;
+}
+
+extern "C" int fs2moe_grouped_swiglu_keep(const void* xe, const int32_t* row_map,
+                                          const int32_t* counts, const int32_t* offsets,
+                                          const void* w_gate, const void* w_up, const void* w_down,
+                                          int32_t E, int32_t D, int32_t F, int64_t max_rows,
+                                          int32_t act_dtype, void* g, void* u, void* h, void* ye,
+                                          void* stream) {
+  FS2_REQUIRE(xe && counts && offsets && w_gate && w_up && w_down && g && u && h && ye,
+              "grouped_swiglu_keep: null pointer");
+  FS2_REQUIRE(E >= 1 && E <= FS2MOE_MAX_EXPERTS, "grouped_swiglu_keep: E=%d outside [1, %d]", E,
+              FS2MOE_MAX_EXPERTS);
+  FS2_REQUIRE(max_rows >= 0 && max_rows < (1ll << 31), "grouped_swiglu_keep: max_rows=%lld",
+              (long long)max_rows);
+  if (!fs2moe_grouped_swiglu_keeps(D, F, max_rows, act_dtype)) {
+    set_error("grouped_swiglu_keep: needs bf16, D and F multiples of 64 and activation matrices "
+              "below 4 GB (D=%d, F=%d, act_dtype %d, max_rows=%lld)",
+              D, F, act_dtype, (long long)max_rows);
+    return FS2MOE_ERR_UNSUPPORTED;
+  }
+  FS2_REQUIRE(aligned16(xe) && aligned16(w_gate) && aligned16(w_up) && aligned16(w_down) &&
+                  aligned16(g) && aligned16(u) && aligned16(h) && aligned16(ye),
+              "grouped_swiglu_keep: buffers must be 16-byte aligned");
+  Groups grp{counts, offsets, E, 0};
+  return launch_dma_pair<FS2MOE_W_IN_OUT>(xe, row_map, grp, max_rows, w_gate, w_up, w_down, nullptr,
+                                          nullptr, nullptr, D, F, h, ye,
+                                          static_cast<hipStream_t>(stream), g, u);
 }
 
 extern "C" int fs2moe_grouped_swiglu(const void* xe, const int32_t* row_map, const int32_t* counts,

@@ -108,7 +108,11 @@ struct TileOrder {
 // of bf16; the producers turn the codes into bf16 in registers (exact) on the way to LDS and lay
 // them out as in the second case, so the consumers' main loop is the same, and the scales multiply
 // the f32 accumulators in the epilogue.
-template <bool DUAL, int BLAYOUT>
+// KEEP_GU (with DUAL, bf16 weights): the epilogue also stores the two products themselves, rounded
+// to bf16 and laid out like C, for a backward pass that would otherwise compute them again.  Their
+// destinations arrive in S0 and S1, which bf16 weights leave unused: two more arguments cost every
+// other variant of the kernel registers in its main loop (1-2.5 % of the layer, measured).
+template <bool DUAL, int BLAYOUT, bool KEEP_GU = false>
 __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     const uint16_t* __restrict__ A, const int32_t* __restrict__ row_map, int lda,
     const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
@@ -116,6 +120,7 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     int Kdim, int N, Groups g, int n_tiles) {
   using namespace dma;
   constexpr bool FP8 = BLAYOUT == W_FP8_TILED;
+  static_assert(!KEEP_GU || (DUAL && !FP8), "the products are kept by the bf16 gate/up kernel only");
   constexpr int BN = DUAL ? 128 : 256;    // real channels per tile
   constexpr int BROW = DUAL ? 256 : 512;  // bytes per LDS row of a weight sub-tile (in x out)
   constexpr bool KN = BLAYOUT == FS2MOE_W_IN_OUT;
@@ -578,6 +583,43 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
       }
     }
   };
+  // KEEP_GU: the same walk twice more, for the gate and the up product (a function of its own so
+  // that the other variants' epilogue compiles to what it was).
+  auto store_products = [&](const Tile& t, int gu) {
+    constexpr int ROWB = 128, CH = 8, RPI = 8;
+    uint8_t* buf = smem_raw + (gu & 1) * UNIT_BYTES + wave * 8192;
+    const uint32_t wbase = (uint32_t)(lr * ROWB + (((lr >> 1) & 7) << 4) + lk * 8);
+    const uint32_t rbase = (uint32_t)((lane / CH) * ROWB + (((lane % CH) ^ (lane >> 4)) << 4));
+    const int n = t.n0 + wn * 64 + (lane % CH) * 8;
+    const int m_wave = t.row0 + wm * 64;
+    const int r_lane = lane / CH;
+    const uint32_t lane_off = (uint32_t)((r_lane * ldc + n) * 2);
+    const bool col_ok = n < N;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+      uint16_t* out = reinterpret_cast<uint16_t*>(const_cast<float*>(which == 0 ? S0 : S1));
+#pragma unroll
+      for (int fm = 0; fm < 2; ++fm) {
+#pragma unroll
+        for (int fn = 0; fn < 2; ++fn)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x16& a = acc[fn + 2 * which][fm];
+            u32x2 o = {pack_bf16x2(a[4 * q], a[4 * q + 1]), pack_bf16x2(a[4 * q + 2], a[4 * q + 3])};
+            *reinterpret_cast<u32x2*>(buf + (wbase ^ (uint32_t)((4 * fn + q) << 4))) = o;
+          }
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) {
+          const u32x4 val = *reinterpret_cast<const u32x4*>(
+              buf + (rbase ^ (uint32_t)((it & 1) << 6)) + it * RPI * ROWB);
+          const int r = m_wave + fm * 32 + it * RPI;  // uniform
+          uint8_t* row_base = reinterpret_cast<uint8_t*>(out + (size_t)r * ldc);
+          if (col_ok && r + r_lane < t.row_end)
+            __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(row_base + lane_off));
+        }
+      }
+    }
+  };
 
   // ---- main stream -----------------------------------------------------------------------------------
   TileOrder order(my_heavy, my_tiles - my_heavy, (int)(blockIdx.x & 7));
@@ -598,6 +640,8 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     if (++ku == nu) {
       __syncthreads();  // every consumer is done with the ring half the epilogue borrows
       if (wave_active) store_tile(cur, gu, tiles_done & 1);
+      if constexpr (KEEP_GU)
+        if (wave_active) store_products(cur, gu);
       ++tiles_done;
       ku = 0;
       if (tiles_left-- > 0) {

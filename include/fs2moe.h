@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FS2MOE_ABI_VERSION 8
+#define FS2MOE_ABI_VERSION 9
 
 /* element types */
 #define FS2MOE_F32 0
@@ -280,6 +280,23 @@ int fs2moe_forward_static(const void* x, const void* residual, const void* route
 int fs2moe_grouped_gemm(const void* a, const int32_t* row_map, const int32_t* counts,
                         const int32_t* offsets, const void* b, int32_t b_layout, int32_t E, int32_t K,
                         int32_t N, int64_t max_rows, int32_t dtype, void* c, void* stream);
+
+/*
+ * fs2moe_grouped_swiglu for the forward pass of a training step: also stores the two products
+ * g = xe @ W_gate and u = xe @ W_up (rounded to the activation dtype), which autograd keeps for the
+ * backward pass of ffn.py:374-395 / experts.py:107-112 (the inputs of SiLU and of the product).
+ * The backward pass can compute them again with two fs2moe_grouped_gemm calls instead; keeping them
+ * costs 2 * rows * F elements of memory and saves those two products.
+ *   bf16 activations and weights (reference layout), D and F multiples of 64, activation matrices
+ *   below 4 GB: fs2moe_grouped_swiglu_keeps says 1; otherwise FS2MOE_ERR_UNSUPPORTED.
+ *   g, u [max_rows, F] (out); everything else as for fs2moe_grouped_swiglu.
+ */
+int fs2moe_grouped_swiglu_keeps(int32_t D, int32_t F, int64_t max_rows, int32_t act_dtype);
+int fs2moe_grouped_swiglu_keep(const void* xe, const int32_t* row_map, const int32_t* counts,
+                               const int32_t* offsets, const void* w_gate, const void* w_up,
+                               const void* w_down, int32_t E, int32_t D, int32_t F,
+                               int64_t max_rows, int32_t act_dtype, void* g, void* u, void* h,
+                               void* ye, void* stream);
 
 /*
  * Weight gradient: dw_e [M, N] = A_e^T @ B_e, the contraction running over the rows of expert e

@@ -84,6 +84,65 @@ def test_grouped_gemm_both_orientations(gpu_device, dtype, layout, rows, k, n):
     assert_grad_close(d, a.double() @ b[0].double(), dtype, "dense")
 
 
+@pytest.mark.parametrize("rows,d,f", [([5, 0, 300, 64, 1, 700], 128, 192), ([130, 257], 64, 64), ([0, 0, 9], 256, 128)])
+def test_grouped_swiglu_keep_leaves_the_two_products(gpu_device, rows, d, f):
+    """The training-forward variant of the expert kernel: same ``ye`` and ``h`` as the inference
+    one, bit for bit, plus the gate and the up product as two separate GEMMs give them."""
+    _say("grouped_swiglu_keep", rows, d, f)
+    dev = gpu_device
+    g = torch.Generator().manual_seed(d + f)
+    e = len(rows)
+    counts, offsets = _groups(rows)
+    total = int(offsets[-1])
+    assert _abi.keeps_products(d, f, total, torch.bfloat16)
+    assert not _abi.keeps_products(d, f, total, torch.float32)
+    assert not _abi.keeps_products(d + 8, f, total, torch.bfloat16)
+    x = torch.randn(total, d, generator=g).to(torch.bfloat16).to(dev)
+    wg, wu = ((0.2 * torch.randn(e * d, f, generator=g)).to(torch.bfloat16).to(dev) for _ in range(2))
+    wd = (0.2 * torch.randn(e * f, d, generator=g)).to(torch.bfloat16).to(dev)
+    c, o = counts.to(dev), offsets.to(dev)
+    ye0, h0 = _abi.grouped_swiglu(x, c, o, wg, wu, wd, e)
+    ye, h, gate, up = _abi.grouped_swiglu_keep(x, c, o, wg, wu, wd, e)
+    gate_ref = _abi.grouped_gemm(x, wg, _abi.W_IN_OUT, c, o, e)
+    up_ref = _abi.grouped_gemm(x, wu, _abi.W_IN_OUT, c, o, e)
+    for ex in range(e):
+        lo, cnt = int(offsets[ex]), int(counts[ex])
+        sl = slice(lo, lo + cnt)
+        assert torch.equal(ye[sl], ye0[sl]) and torch.equal(h[sl], h0[sl]), f"expert {ex}: ye / h differ"
+        assert torch.equal(gate[sl], gate_ref[sl]), f"expert {ex}: gate product"
+        assert torch.equal(up[sl], up_ref[sl]), f"expert {ex}: up product"
+        if cnt:
+            ref = x[sl].double().cpu() @ wg.double().cpu().reshape(e, d, f)[ex]
+            assert_grad_close(gate[sl], ref, "bf16", f"expert {ex} gate product")
+    # through a row map
+    perm = torch.randperm(total, generator=g).to(torch.int32)
+    xs = torch.empty_like(x)
+    xs[perm.long().to(dev)] = x
+    ye2, _, gate2, up2 = _abi.grouped_swiglu_keep(xs, c, o, wg, wu, wd, e, row_map=perm.to(dev))
+    for ex in range(e):
+        sl = slice(int(offsets[ex]), int(offsets[ex]) + int(counts[ex]))
+        assert torch.equal(ye2[sl], ye0[sl]) and torch.equal(gate2[sl], gate[sl]) and torch.equal(up2[sl], up[sl])
+
+
+def test_backward_twice_gives_the_same_gradients(gpu_device):
+    """The kept products are autograd's saved tensors: a backward pass must leave them as they are
+    (``retain_graph=True`` and a second pass is how a trainer accumulates two losses)."""
+    wl = W.make_workload_from_spec(W.small_spec(dtype="bf16", tokens=96, num_experts=8, model_dim=128, inner_dim=128, seed=5))
+    m = build_module(wl, gpu_device).train().requires_grad_(True)
+    x = wl.x.to(torch.bfloat16).to(gpu_device).requires_grad_(True)
+    out = m(x)
+    go = torch.randn_like(out)
+    out.backward(go, retain_graph=True)
+    first = [x.grad.clone()] + [p.grad.clone() for p in m.parameters()]
+    x.grad = None
+    for p in m.parameters():
+        p.grad = None
+    out.backward(go)
+    second = [x.grad] + [p.grad for p in m.parameters()]
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
 @pytest.mark.parametrize("rows,m,n", [([5, 0, 300, 64, 1], 64, 96), ([130, 257], 136, 264), ([33], 8, 8), ([0, 0], 128, 128)])
 def test_grouped_wgrad_matches_torch(gpu_device, dtype, rows, m, n):
