@@ -10,6 +10,8 @@
 //   * router_backward_kernel combine-weight gradients -> logit gradients (sigmoid / softmax, with
 //                            or without renormalisation over the selected experts)
 // They are what torch.autograd derives from moe.py:102-157, experts.py:102-112 and ffn.py:374-395.
+#include <type_traits>
+
 #include "common.h"
 #include "tile_map.h"
 
@@ -21,15 +23,18 @@ namespace fs2moe {
 // rows RK at a time (32 for bf16, 16 for f32).  Both chunks go to LDS as they lie in memory (row =
 // contraction index, columns contiguous) and come back through the transposing LDS read (bf16) or
 // as single floats (f32), each already in MFMA operand order.  LDS holds two chunks: while one is
-// multiplied the next is written from registers and the one after that is on its way from memory,
-// so there is one barrier per chunk.  Rows past the expert's count are zero-filled, experts without
-// rows get a zero gradient.
+// multiplied the next is written from registers and the two after that are on their way from memory
+// in two sets of registers, so there is one barrier per chunk, which orders LDS traffic only.  Rows
+// past the expert's count are zero-filled, experts without rows get a zero gradient.
 namespace wgk {
 constexpr int TM = 256, TN = 256, WAVES = 8;
 constexpr int SMEM_BYTES = 65536;  // two chunks of both operands
 }
 
-template <typename T>
+// MAPPED: A's rows are read through a_map.  A template parameter, not a test of the pointer: behind
+// a condition the map entry's load is waited for with every other load of the wave (the counter
+// cannot tell them apart at the join), which serialises a chunk's loads into round trips.
+template <typename T, bool MAPPED>
 __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
     const T* __restrict__ A, const int32_t* __restrict__ a_map, int lda, const T* __restrict__ B,
     int ldb, T* __restrict__ C, int M, int N, Groups g, int m_tiles, int n_tiles, int seg_rows,
@@ -97,26 +102,40 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
   // Loads are unconditional, from clamped addresses (a select behind a load would make the wave wait
   // for it at once); what lies past the expert's rows or the matrix's columns is zeroed when the
   // registers go to LDS.
-  u32x4 ra[PER_THREAD], rb[PER_THREAD];
-  bool va[PER_THREAD], vb[PER_THREAD];
+  // Two sets of registers, so that two chunks are on their way from memory at any time (one chunk's
+  // loads take about as long as its MFMAs do: with a single set every chunk waited for its loads).
+  u32x4 ra[2][PER_THREAD], rb[2][PER_THREAD];
+  bool va[2][PER_THREAD], vb[2][PER_THREAD];
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
-  auto load_chunk = [&](int r0) {
+  auto load_chunk = [&](auto set_c, int r0) {
+    constexpr int set = decltype(set_c)::value;
+    int rr[PER_THREAD], arow[PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int r = r0 + (tid + WAVES * 64 * i) / ROW_CHUNKS;
+      rr[i] = off + (r < cnt ? r : cnt - 1);  // cnt > 0 here
+      arow[i] = rr[i];
+    }
+    if constexpr (MAPPED) {  // all the map entries first, then all the rows
+#pragma unroll
+      for (int i = 0; i < PER_THREAD; ++i) arow[i] = a_map[rr[i]];
+    }
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
       const int c = tid + WAVES * 64 * i;
       const int k = c / ROW_CHUNKS, ch = c % ROW_CHUNKS;
-      const int r = r0 + k;
-      const bool row_ok = r < cnt;
-      const int rr = off + (row_ok ? r : cnt - 1);  // cnt > 0 here
-      const int arow = a_map != nullptr ? a_map[rr] : rr;
+      const bool row_ok = r0 + k < cnt;
       const bool a_ok = m0 + ch * VEC < M, b_ok = n0 + ch * VEC < N;
-      va[i] = row_ok && a_ok;
-      vb[i] = row_ok && b_ok;
-      ra[i] = *reinterpret_cast<const u32x4*>(A + (size_t)arow * lda + (a_ok ? m0 + ch * VEC : 0));
-      rb[i] = *reinterpret_cast<const u32x4*>(B + (size_t)rr * ldb + (b_ok ? n0 + ch * VEC : 0));
+      va[set][i] = row_ok && a_ok;
+      vb[set][i] = row_ok && b_ok;
+      ra[set][i] =
+          *reinterpret_cast<const u32x4*>(A + (size_t)arow[i] * lda + (a_ok ? m0 + ch * VEC : 0));
+      rb[set][i] =
+          *reinterpret_cast<const u32x4*>(B + (size_t)rr[i] * ldb + (b_ok ? n0 + ch * VEC : 0));
     }
   };
-  auto store_chunk = [&](int buf) {
+  auto store_chunk = [&](auto set_c, int buf) {
+    constexpr int set = decltype(set_c)::value;
     uint8_t* sA = smem + buf * 2 * OPB;
     uint8_t* sB = sA + OPB;
 #pragma unroll
@@ -126,8 +145,8 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
       // bf16: chunk ch of row k sits in slot ch ^ ((k & 3) << 2), so that the four consecutive rows
       // a transposing read touches lie 64 bytes apart
       const int slot = BF16 ? (ch ^ ((k & 3) << 2)) : ch;
-      *reinterpret_cast<u32x4*>(sA + k * ROWB + slot * 16) = va[i] ? ra[i] : zero4;
-      *reinterpret_cast<u32x4*>(sB + k * ROWB + slot * 16) = vb[i] ? rb[i] : zero4;
+      *reinterpret_cast<u32x4*>(sA + k * ROWB + slot * 16) = va[set][i] ? ra[set][i] : zero4;
+      *reinterpret_cast<u32x4*>(sB + k * ROWB + slot * 16) = vb[set][i] ? rb[set][i] : zero4;
     }
   };
 
@@ -191,21 +210,28 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
     }
   };
 
-  // chunk i is multiplied from LDS buffer i & 1 while chunk i + 1 goes from the registers into the
-  // other buffer (read last during chunk i - 1: the barrier that ended it has passed) and chunk i + 2
-  // is loaded
+  // Chunk i is multiplied from LDS buffer i & 1 while chunk i + 1 goes from register set (i + 1) & 1
+  // into the other buffer (read last during chunk i - 1: the barrier that ended it has passed), chunk
+  // i + 3 is loaded into the set this frees, and chunk i + 2 is still on its way in the other set.
   const int chunks = (cnt + RK - 1) / RK;
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
   if (chunks > 0) {
-    load_chunk(0);
-    store_chunk(0);
-    if (chunks > 1) load_chunk(RK);
+    load_chunk(Set0{}, 0);
+    if (chunks > 1) load_chunk(Set1{}, RK);
+    store_chunk(Set0{}, 0);
+    if (chunks > 2) load_chunk(Set0{}, 2 * RK);
     __syncthreads();
   }
-  for (int i = 0; i < chunks; ++i) {
-    if (i + 1 < chunks) store_chunk((i + 1) & 1);
-    if (i + 2 < chunks) load_chunk((i + 2) * RK);
+  auto step = [&](int i, auto next_set) {
+    if (i + 1 < chunks) store_chunk(next_set, (i + 1) & 1);
+    if (i + 3 < chunks) load_chunk(next_set, (i + 3) * RK);
     compute_chunk(i & 1);
-    __syncthreads();
+    lds_barrier();  // the loads of the next chunks stay in flight
+  };
+  for (int i = 0; i < chunks; i += 2) {
+    step(i, Set1{});
+    if (i + 1 < chunks) step(i + 1, Set0{});
   }
 
   // Accumulator layout: the lane holds row m = lr of fragment tm and columns 8 q + 4 lk + {0..3} of
@@ -507,18 +533,22 @@ extern "C" int fs2moe_grouped_wgrad(const void* a, const int32_t* a_row_map, con
   FS2_REQUIRE(blocks <= 0x7fffffffll, "grouped_wgrad: too many tiles");
   Groups g{counts, offsets, E, (int)max_rows};
   hipStream_t st = static_cast<hipStream_t>(stream);
-  auto kb = grouped_wgrad_kernel<uint16_t>;
-  auto kf = grouped_wgrad_kernel<float>;
+  const bool mapped = a_row_map != nullptr;
+  auto kb = mapped ? grouped_wgrad_kernel<uint16_t, true> : grouped_wgrad_kernel<uint16_t, false>;
+  auto kf = mapped ? grouped_wgrad_kernel<float, true> : grouped_wgrad_kernel<float, false>;
   static bool attr_set = false;  // benign race: setting the attribute is idempotent
   if (!attr_set) {
-    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(kb),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, wgk::SMEM_BYTES);
-    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(kf),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, wgk::SMEM_BYTES);
-    if (e1 != hipSuccess || e2 != hipSuccess) {
-      set_error("grouped_wgrad: cannot reserve %d bytes of LDS: %s", wgk::SMEM_BYTES,
-                hipGetErrorString(e1 != hipSuccess ? e1 : e2));
-      return FS2MOE_ERR_LAUNCH;
+    const void* ks[4] = {reinterpret_cast<const void*>(grouped_wgrad_kernel<uint16_t, false>),
+                         reinterpret_cast<const void*>(grouped_wgrad_kernel<uint16_t, true>),
+                         reinterpret_cast<const void*>(grouped_wgrad_kernel<float, false>),
+                         reinterpret_cast<const void*>(grouped_wgrad_kernel<float, true>)};
+    for (const void* k : ks) {
+      hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, wgk::SMEM_BYTES);
+      if (e != hipSuccess) {
+        set_error("grouped_wgrad: cannot reserve %d bytes of LDS: %s", wgk::SMEM_BYTES,
+                  hipGetErrorString(e));
+        return FS2MOE_ERR_LAUNCH;
+      }
     }
     attr_set = true;
   }

@@ -138,6 +138,14 @@ __device__ __forceinline__ bf16x8 lds_read_frag_tr(const uint16_t* p_lo, const u
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// Block barrier that orders LDS traffic only.  __syncthreads() also fences global memory, for which
+// the compiler drains every outstanding global load (s_waitcnt vmcnt(0)); loops that keep a register
+// set of loads in flight across their barriers, and synchronise on nothing that lives in global
+// memory, use this one.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // 8 e4m3 codes (two dwords) -> 8 bf16 values.
 __device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(uint32_t lo, uint32_t hi) {
   typedef __attribute__((ext_vector_type(2))) float f32x2;

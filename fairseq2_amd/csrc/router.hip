@@ -343,14 +343,6 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_fma_kernel(
   }
 }
 
-// Block barrier that orders LDS traffic only.  __syncthreads() also fences global memory, for which
-// the compiler drains every outstanding global load (s_waitcnt vmcnt(0)); the router loops keep a
-// register set of loads in flight across their barriers, and nothing they synchronise on lives in
-// global memory.
-__device__ __forceinline__ void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
 // ----------------------------------------------------------------------------------- bf16 / MFMA
 namespace rmfma {
 constexpr int BT = 32;      // tokens per block (one MFMA tile wide)
