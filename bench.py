@@ -284,7 +284,7 @@ def main() -> int:
 
     import torch
 
-    from fairseq2_amd import workloads as W
+    import workloads as W
 
     if not torch.cuda.is_available():
         print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)

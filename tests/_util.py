@@ -5,8 +5,8 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from fairseq2_amd import workloads as W
-from fairseq2_amd.workloads import build_module  # noqa: F401
+import workloads as W
+from workloads import build_module  # noqa: F401
 from oracle import moe_oracle as O
 
 TORCH_DTYPE = {"fp32": torch.float32, "bf16": torch.bfloat16}

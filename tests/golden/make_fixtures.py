@@ -30,7 +30,7 @@ import torch
 HERE = Path(__file__).resolve().parent
 sys.path.insert(0, str(HERE.parent.parent))
 
-from fairseq2_amd import workloads as W  # noqa: E402
+import workloads as W  # noqa: E402
 from oracle import moe_oracle as O  # noqa: E402
 
 # name -> (spec keywords, number of leading tokens whose input row is zeroed: all their logits tie)

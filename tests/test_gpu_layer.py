@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from fairseq2_amd import _abi
-from fairseq2_amd import workloads as W
+import workloads as W
 from oracle import moe_oracle as O
 from tests._util import (
     TORCH_DTYPE, assert_output_close, assert_routing_equal, build_module, oracle_forward, oracle_routing,

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from fairseq2_amd import _abi
-from fairseq2_amd import workloads as W
+import workloads as W
 from oracle import moe_oracle as O
 from tests._util import TORCH_DTYPE, assert_output_close, assert_routing_equal, oracle_routing
 

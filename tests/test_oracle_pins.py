@@ -487,7 +487,7 @@ def test_bf16_rounding_budget_of_the_device_pipeline():
     overall error is a few tenths of a percent of the output's rms, well inside RMS_TOL, and every
     element is inside the element-wise bound with room to spare (the largest errors sit on the largest
     elements, where the final rounding alone is 2^-9 of the value: they are what rtol is for)."""
-    from fairseq2_amd import workloads as W
+    import workloads as W
     from tests._util import RMS_TOL, TOL, emulate_device_rounding, oracle_forward, oracle_routing
 
     spec = W.small_spec(tokens=300, model_dim=256, num_experts=16, top_k=16, inner_dim=192, dtype="bf16",

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from fairseq2_amd import workloads as W
+import workloads as W
 from oracle import moe_oracle as O
 
 

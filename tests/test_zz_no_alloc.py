@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from fairseq2_amd import _abi
-from fairseq2_amd import workloads as W
+import workloads as W
 from fairseq2_amd.moe import _SCORE_FNS
 from tests._util import TORCH_DTYPE, build_module
 
