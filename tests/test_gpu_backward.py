@@ -124,6 +124,50 @@ def test_grouped_swiglu_keep_leaves_the_two_products(gpu_device, rows, d, f):
         assert torch.equal(ye2[sl], ye0[sl]) and torch.equal(gate2[sl], gate[sl]) and torch.equal(up2[sl], up[sl])
 
 
+def test_full_size_weight_gradient_and_kept_products(gpu_device):
+    """The Qwen3 prefill shape's own routing (65536 rows over 128 experts, from none to thousands of
+    rows each): the weight gradient and the kept products of sampled experts against torch's f32
+    matmul on the same device, every empty expert's gradient exactly zero."""
+    wl = W.make_workload("qwen3_30b_a3b", with_weights=False)
+    spec = wl.spec
+    dev = gpu_device
+    d, f, e = spec.model_dim, spec.inner_dim, spec.num_experts
+    x = wl.x.reshape(-1, d).to(torch.bfloat16).to(dev)
+    m = spec.mode
+    idx, w, _ = _abi.router_topk(x, wl.router.to(torch.bfloat16).to(dev), wl.router_bias.to(dev), spec.top_k,
+                                 _abi.SCORE_SOFTMAX if m.score_fn == "softmax" else _abi.SCORE_SIGMOID,
+                                 m.renormalize, want_logits=True)
+    disp = _abi.dispatch(idx, w, x, e, 16, False, gather=True)
+    counts, offsets = disp.counts.cpu(), disp.offsets.cpu()
+    rows = disp.xe.shape[0]
+    g = torch.Generator().manual_seed(11)
+    dy = torch.randn(rows, f, generator=g).to(torch.bfloat16).to(dev)
+    dw = _abi.grouped_wgrad(disp.xe, dy, disp.counts, disp.offsets, e).view(e, d, f)
+    order = torch.argsort(counts, descending=True)
+    sample = [int(order[0]), int(order[len(order) // 4]), int(order[len(order) // 2])]
+    sample += [int(i) for i in torch.nonzero(counts > 0).flatten()[-2:]]
+    for ex in sample:
+        lo, cnt = int(offsets[ex]), int(counts[ex])
+        ref = disp.xe[lo : lo + cnt].float().t() @ dy[lo : lo + cnt].float()
+        _say(f"  expert {ex}: {cnt} rows")
+        assert_grad_close(dw[ex], ref.double().cpu(), "bf16", f"weight gradient of expert {ex} ({cnt} rows)")
+    for ex in torch.nonzero(counts == 0).flatten().tolist():
+        assert not bool(dw[ex].any()), f"expert {ex} has no rows but a gradient"
+    # the kept products of the training forward
+    wg, wu = ((0.05 * torch.randn(e * d, f, generator=g)).to(torch.bfloat16).to(dev) for _ in range(2))
+    wd = (0.05 * torch.randn(e * f, d, generator=g)).to(torch.bfloat16).to(dev)
+    ye, h, gate, up = _abi.grouped_swiglu_keep(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
+    ye0, h0 = _abi.grouped_swiglu(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
+    for ex in sample:
+        lo, cnt = int(offsets[ex]), int(counts[ex])
+        sl = slice(lo, lo + cnt)
+        assert torch.equal(ye[sl], ye0[sl]) and torch.equal(h[sl], h0[sl])
+        ref = disp.xe[sl].float() @ wg.view(e, d, f)[ex].float()
+        assert_grad_close(gate[sl], ref.double().cpu(), "bf16", f"gate product of expert {ex}")
+        ref = disp.xe[sl].float() @ wu.view(e, d, f)[ex].float()
+        assert_grad_close(up[sl], ref.double().cpu(), "bf16", f"up product of expert {ex}")
+
+
 def test_backward_twice_gives_the_same_gradients(gpu_device):
     """The kept products are autograd's saved tensors: a backward pass must leave them as they are
     (``retain_graph=True`` and a second pass is how a trainer accumulates two losses)."""
