@@ -15,7 +15,7 @@ from torch import Tensor
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfs2moe.so")
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
@@ -56,6 +56,10 @@ _PROTOTYPES = {
     ),
     "fs2moe_grouped_swiglu_fuses_gather": (c_int32, [c_int32, c_int32, c_int32, c_int32]),
     "fs2moe_grouped_swiglu_keeps": (c_int32, [c_int32, c_int32, c_int64, c_int32]),
+    "fs2moe_grouped_gemm_sum_supported": (c_int32, [c_int32, c_int32, c_int64, c_int32]),
+    "fs2moe_grouped_gemm_sum": (
+        c_int32, [c_void_p] * 6 + [c_int32] * 3 + [c_int64, c_int32, c_void_p, c_void_p],
+    ),
     "fs2moe_grouped_swiglu_keep": (
         c_int32,
         [c_void_p] * 7 + [c_int32] * 3 + [c_int64, c_int32] + [c_void_p] * 5,
@@ -553,6 +557,42 @@ def grouped_gemm(
         dtype_code(a.dtype), _ptr(c), _stream(),
     )
     _check(rc, "fs2moe_grouped_gemm")
+    return c
+
+
+def grouped_gemm_sum_supported(k: int, n: int, rows: int, dtype: torch.dtype) -> bool:
+    """Whether :func:`grouped_gemm_sum` exists for these sizes and this type."""
+    return bool(load().fs2moe_grouped_gemm_sum_supported(k, n, rows, dtype_code(dtype)))
+
+
+def grouped_gemm_sum(
+    a1: Tensor, b1: Tensor, a2: Tensor, b2: Tensor,
+    counts: Tensor | None = None, offsets: Tensor | None = None, num_experts: int = 1,
+) -> Tensor:
+    """``c[r] = a1[r] @ B1_e^T + a2[r] @ B2_e^T`` with ``(E*N, K)`` weights, one rounding
+    (``fs2moe_grouped_gemm_sum``)."""
+    lib = load()
+    e = num_experts
+    rows, k = a1.shape
+    n = b1.shape[0] // e
+    _same("a2", a2, (rows, k), a1.dtype, a1.device)
+    _same("b1", b1, (e * n, k), a1.dtype, a1.device)
+    _same("b2", b2, (e * n, k), a1.dtype, a1.device)
+    if not a1.is_contiguous():
+        raise ValueError("a1 must be contiguous")
+    if (counts is None) != (offsets is None):
+        raise ValueError("counts and offsets come together")
+    if counts is not None:
+        _same("counts", counts, (e,), torch.int32, a1.device)
+        _same("offsets", offsets, (e + 1,), torch.int32, a1.device)
+    elif e != 1:
+        raise ValueError("a dense product has one matrix")
+    c = torch.empty((rows, n), dtype=a1.dtype, device=a1.device)
+    rc = lib.fs2moe_grouped_gemm_sum(
+        _ptr(a1), _ptr(b1), _ptr(a2), _ptr(b2), _ptr(counts), _ptr(offsets), e, k, n, rows,
+        dtype_code(a1.dtype), _ptr(c), _stream(),
+    )
+    _check(rc, "fs2moe_grouped_gemm_sum")
     return c
 
 

@@ -14,7 +14,8 @@ derivation is written out once, against ``moe.py:102-157``, ``experts.py:102-112
                                                 or computed again               -> fs2moe_grouped_gemm
     dg, du   = SwiGLU'(g, u, dh),  h = SiLU(g) u                               -> fs2moe_swiglu_backward
     dWd, dWg, dWu = h^T dye, xe^T dg, xe^T du  per expert                      -> fs2moe_grouped_wgrad
-    dxe      = dg @ Wg^T + du @ Wu^T                                           -> fs2moe_grouped_gemm
+    dxe      = dg @ Wg^T + du @ Wu^T                                           -> fs2moe_grouped_gemm_sum
+                                                                                  (or two fs2moe_grouped_gemm)
     dw       = <ye, dout[token]>  or  <dxe, x[token]>                          -> fs2moe_pair_dot
     dlogits  = score'(logits) dw                                               -> fs2moe_router_backward
     drouter  = x^T dlogits,  dx += dlogits @ router^T                          -> wgrad / gemm, one group
@@ -73,8 +74,13 @@ def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
     d_wd = _abi.grouped_wgrad(h, dye, **grp) if need[4] else None
     d_wg = _abi.grouped_wgrad(xe, dg, **grp) if need[2] else None
     d_wu = _abi.grouped_wgrad(xe, du, **grp) if need[3] else None
-    dxe_g = _abi.grouped_gemm(dg, wg, OUT_IN, **grp)
-    dxe_u = _abi.grouped_gemm(du, wu, OUT_IN, **grp)
+    # dxe = dg @ Wg^T + du @ Wu^T: one kernel and one rounding where the library has it, else the
+    # two products apart (their sum is then taken where dxe is used)
+    if _abi.grouped_gemm_sum_supported(dg.shape[1], x.shape[1], dg.shape[0], dg.dtype):
+        dxe_g, dxe_u = _abi.grouped_gemm_sum(dg, wg, du, wu, **grp), None
+    else:
+        dxe_g = _abi.grouped_gemm(dg, wg, OUT_IN, **grp)
+        dxe_u = _abi.grouped_gemm(du, wu, OUT_IN, **grp)
 
     # combine weights -> logits -> router and x
     if scale_input:
@@ -103,8 +109,11 @@ def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
         # shared expert): two scatter passes, one per half of dxe, each starting from up to two dense
         # rows (the kernel's base and residual operands), everything summed in f32
         dense = dx_parts + [None] * (3 - len(dx_parts))
+        if dxe_u is None and dense[2] is not None:
+            dense = [dense[0] + dense[1], dense[2], None]  # one pass takes two dense terms
         t1 = _abi.combine(dxe_g, inv_perm, idx, w, dense[0], scale_input, residual=dense[1])
-        dx = _abi.combine(dxe_u, inv_perm, idx, w, t1, scale_input, out=t1, residual=dense[2])
+        dx = t1 if dxe_u is None else _abi.combine(dxe_u, inv_perm, idx, w, t1, scale_input, out=t1,
+                                                   residual=dense[2])
     return dx, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd
 
 

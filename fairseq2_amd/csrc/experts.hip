@@ -678,6 +678,66 @@ extern "C" int fs2moe_grouped_gemm(const void* a, const int32_t* row_map, const 
   return launch_gemm<FS2MOE_W_OUT_IN>(a, row_map, g, max_rows, b, K, N, dtype, c, st);
 }
 
+extern "C" int fs2moe_grouped_gemm_sum_supported(int32_t K, int32_t N, int64_t max_rows,
+                                                 int32_t dtype) {
+  if (K <= 0 || N <= 0 || max_rows < 0 || N % 8 != 0) return 0;
+  return (dtype == FS2MOE_BF16 && K % (2 * dma::BK) == 0 && dma_offsets_fit(max_rows, K, N)) ? 1 : 0;
+}
+
+extern "C" int fs2moe_grouped_gemm_sum(const void* a1, const void* b1, const void* a2,
+                                       const void* b2, const int32_t* counts,
+                                       const int32_t* offsets, int32_t E, int32_t K, int32_t N,
+                                       int64_t max_rows, int32_t dtype, void* c, void* stream) {
+  FS2_REQUIRE(a1 && b1 && a2 && b2 && c, "grouped_gemm_sum: null pointer");
+  FS2_REQUIRE((counts == nullptr) == (offsets == nullptr),
+              "grouped_gemm_sum: counts without offsets");
+  FS2_REQUIRE(E >= 1 && E <= FS2MOE_MAX_EXPERTS && (counts != nullptr || E == 1),
+              "grouped_gemm_sum: E=%d", E);
+  FS2_REQUIRE(max_rows >= 0 && max_rows < (1ll << 31), "grouped_gemm_sum: max_rows=%lld",
+              (long long)max_rows);
+  if (!fs2moe_grouped_gemm_sum_supported(K, N, max_rows, dtype)) {
+    set_error("grouped_gemm_sum: needs bf16, K a multiple of 64, N a multiple of 8 and matrices "
+              "below 4 GB (K=%d, N=%d, dtype %d, max_rows=%lld)",
+              K, N, dtype, (long long)max_rows);
+    return FS2MOE_ERR_UNSUPPORTED;
+  }
+  FS2_REQUIRE(aligned16(a1) && aligned16(b1) && aligned16(a2) && aligned16(b2) && aligned16(c),
+              "grouped_gemm_sum: buffers must be 16-byte aligned");
+  if (max_rows == 0) return FS2MOE_OK;
+  using namespace dma;
+  Groups g{counts, offsets, E, (int)max_rows};
+  auto k = glu_gemm_bf16_dma_kernel<false, FS2MOE_W_OUT_IN, false, true>;
+  static bool attr_set = false;  // benign race: setting the attribute is idempotent
+  if (!attr_set) {
+    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(k),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+    if (e1 != hipSuccess) {
+      set_error("grouped_gemm_sum: cannot reserve %d bytes of LDS: %s", SMEM_BYTES,
+                hipGetErrorString(e1));
+      return FS2MOE_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  const int num_blocks = cu_count_by_xcd();
+  if (num_blocks == 0) {
+    set_error("grouped_gemm_sum: cannot query the compute-unit count");
+    return FS2MOE_ERR_LAUNCH;
+  }
+  const int groups = counts ? E : 0;
+  const int nt = (N + 255) / 256;
+  if ((max_rows / BM + groups + 1) * nt > 0x7fffffffll) {
+    set_error("grouped_gemm_sum: too many tiles");
+    return FS2MOE_ERR_UNSUPPORTED;
+  }
+  // (the second activation matrix travels in the first scale argument, the second weights in B1)
+  hipLaunchKernelGGL(k, dim3((unsigned)num_blocks), dim3(NWAVES * 64), SMEM_BYTES,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(a1),
+                     static_cast<const int32_t*>(nullptr), K, static_cast<const uint16_t*>(b1),
+                     static_cast<const uint16_t*>(b2), static_cast<const float*>(a2),
+                     static_cast<const float*>(nullptr), static_cast<uint16_t*>(c), N, K, N, g, nt);
+  return check_launch("glu_gemm_bf16_dma<two sources>");
+}
+
 extern "C" int fs2moe_dense_swiglu(const void* x, const void* w_gate, const void* w_up,
                                    const void* w_down, int32_t T, int32_t D, int32_t F,
                                    int32_t act_dtype, void* h, void* y, void* stream) {

@@ -112,7 +112,10 @@ struct TileOrder {
 // to bf16 and laid out like C, for a backward pass that would otherwise compute them again.  Their
 // destinations arrive in S0 and S1, which bf16 weights leave unused: two more arguments cost every
 // other variant of the kernel registers in its main loop (1-2.5 % of the layer, measured).
-template <bool DUAL, int BLAYOUT, bool KEEP_GU = false>
+// TWO_SRC (single matrix, (out, in) bf16 weights): C = A @ B0_e^T + A2 @ B1_e^T, the second pair
+// walked after the first into the same accumulators (Kdim is one pair's).  A2 arrives in S0, for the
+// reason given above.
+template <bool DUAL, int BLAYOUT, bool KEEP_GU = false, bool TWO_SRC = false>
 __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     const uint16_t* __restrict__ A, const int32_t* __restrict__ row_map, int lda,
     const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1,
@@ -121,6 +124,7 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
   using namespace dma;
   constexpr bool FP8 = BLAYOUT == W_FP8_TILED;
   static_assert(!KEEP_GU || (DUAL && !FP8), "the products are kept by the bf16 gate/up kernel only");
+  static_assert(!TWO_SRC || (!DUAL && BLAYOUT == FS2MOE_W_OUT_IN), "two sources: one (out, in) matrix each");
   constexpr int BN = DUAL ? 128 : 256;    // real channels per tile
   constexpr int BROW = DUAL ? 256 : 512;  // bytes per LDS row of a weight sub-tile (in x out)
   constexpr bool KN = BLAYOUT == FS2MOE_W_IN_OUT;
@@ -198,7 +202,8 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
   const int heavy_end = total_heavy * n_tiles;
   const int my_heavy = slot < heavy_end ? (heavy_end - slot + grid - 1) / grid : 0;
 
-  const int nu = Kdim / (2 * BK);  // units per tile; the host guarantees Kdim % 64 == 0
+  // units per tile; the host guarantees Kdim % 64 == 0
+  const int nu = (TWO_SRC ? 2 : 1) * (Kdim / (2 * BK));
   const int total_units = my_tiles * nu;
 
   // Wave-uniform parameters of a tile: expert, first row, end row, first channel.
@@ -285,7 +290,7 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
         ++ld_tiles;
       } else {
         ld_bg = B0 + (size_t)t.e * wstride;
-        ld_bu = DUAL ? B1 + (size_t)t.e * wstride : ld_bg;
+        ld_bu = (DUAL || TWO_SRC) ? B1 + (size_t)t.e * wstride : ld_bg;
       }
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
@@ -347,7 +352,11 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     float stage_scale = 0.f;
     // Unit ku of the tile set up last -> registers.
     auto load_unit = [&](int ku) {
-      const uint8_t* abase = reinterpret_cast<const uint8_t*>(A + (size_t)ku * (2 * BK));
+      // with two sources the second half of a tile's units comes from the second pair
+      const bool second = TWO_SRC && ku >= nu / 2;
+      if constexpr (TWO_SRC) ku = second ? ku - nu / 2 : ku;
+      const uint16_t* a_src = second ? reinterpret_cast<const uint16_t*>(S0) : A;
+      const uint8_t* abase = reinterpret_cast<const uint8_t*>(a_src + (size_t)ku * (2 * BK));
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj)
         if (jj < a_pieces) stage[jj] = *reinterpret_cast<const u32x4*>(abase + pa[jj]);
@@ -372,8 +381,10 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
           stage[8 + 4 * h + 3] = *reinterpret_cast<const u32x4*>(bu + pb[3]);
         }
       } else {
-        const uint8_t* bg = reinterpret_cast<const uint8_t*>(ld_bg + (size_t)ku * (2 * BK));
-        const uint8_t* bu = reinterpret_cast<const uint8_t*>(ld_bu + (size_t)ku * (2 * BK));
+        const uint8_t* bg =
+            reinterpret_cast<const uint8_t*>((second ? ld_bu : ld_bg) + (size_t)ku * (2 * BK));
+        const uint8_t* bu =
+            TWO_SRC ? bg : reinterpret_cast<const uint8_t*>(ld_bu + (size_t)ku * (2 * BK));
         // pieces q + 4 jj: jj < 4 lie in rows 0..127 (gate when DUAL), the rest in rows 128..255
 #pragma unroll
         for (int jj = 0; jj < 8; ++jj)

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FS2MOE_ABI_VERSION 9
+#define FS2MOE_ABI_VERSION 10
 
 /* element types */
 #define FS2MOE_F32 0
@@ -280,6 +280,19 @@ int fs2moe_forward_static(const void* x, const void* residual, const void* route
 int fs2moe_grouped_gemm(const void* a, const int32_t* row_map, const int32_t* counts,
                         const int32_t* offsets, const void* b, int32_t b_layout, int32_t E, int32_t K,
                         int32_t N, int64_t max_rows, int32_t dtype, void* c, void* stream);
+
+/*
+ * Two grouped GEMMs into one result: c[r] = a1[r] @ B1_e^T + a2[r] @ B2_e^T for the rows r of every
+ * expert e, accumulated in f32 and rounded once.  The input gradient of the gate/up pair of
+ * experts.py:107-112 (x @ gate_proj and x @ inner_proj share x, so their input gradients add).
+ *   a1, a2 [rows, K] bf16; b1, b2 [E*N, K] bf16 (FS2MOE_W_OUT_IN); c [max_rows, N] bf16 (out).
+ *   bf16 only, K a multiple of 64, N of 8, matrices below 4 GB: fs2moe_grouped_gemm_sum_supported
+ *   says 1; otherwise FS2MOE_ERR_UNSUPPORTED (two fs2moe_grouped_gemm calls and an addition do it).
+ */
+int fs2moe_grouped_gemm_sum_supported(int32_t K, int32_t N, int64_t max_rows, int32_t dtype);
+int fs2moe_grouped_gemm_sum(const void* a1, const void* b1, const void* a2, const void* b2,
+                            const int32_t* counts, const int32_t* offsets, int32_t E, int32_t K,
+                            int32_t N, int64_t max_rows, int32_t dtype, void* c, void* stream);
 
 /*
  * fs2moe_grouped_swiglu for the forward pass of a training step: also stores the two products

@@ -84,6 +84,32 @@ def test_grouped_gemm_both_orientations(gpu_device, dtype, layout, rows, k, n):
     assert_grad_close(d, a.double() @ b[0].double(), dtype, "dense")
 
 
+@pytest.mark.parametrize("rows,k,n", [([5, 0, 300, 64, 1, 700], 192, 128), ([130, 257], 64, 72), ([0, 0, 9], 128, 256)])
+def test_grouped_gemm_sum_adds_two_products(gpu_device, rows, k, n):
+    """``a1 @ B1^T + a2 @ B2^T`` in one kernel against f64, and against the two products apart."""
+    _say("grouped_gemm_sum", rows, k, n)
+    dev = gpu_device
+    g = torch.Generator().manual_seed(k * n)
+    e = len(rows)
+    counts, offsets = _groups(rows)
+    total = int(offsets[-1])
+    assert _abi.grouped_gemm_sum_supported(k, n, total, torch.bfloat16)
+    assert not _abi.grouped_gemm_sum_supported(k, n, total, torch.float32)
+    assert not _abi.grouped_gemm_sum_supported(k + 8, n, total, torch.bfloat16)
+    a1, a2 = (torch.randn(total, k, generator=g).to(torch.bfloat16) for _ in range(2))
+    b1, b2 = ((0.1 * torch.randn(e, n, k, generator=g)).to(torch.bfloat16) for _ in range(2))
+    c, o = counts.to(dev), offsets.to(dev)
+    out = _abi.grouped_gemm_sum(a1.to(dev), b1.reshape(e * n, k).to(dev), a2.to(dev), b2.reshape(e * n, k).to(dev), c, o, e)
+    for ex in range(e):
+        lo, cnt = int(offsets[ex]), int(counts[ex])
+        if cnt:
+            ref = a1[lo : lo + cnt].double() @ b1[ex].double().t() + a2[lo : lo + cnt].double() @ b2[ex].double().t()
+            assert_grad_close(out[lo : lo + cnt], ref, "bf16", f"expert {ex}")
+    # one matrix each, all rows
+    dense = _abi.grouped_gemm_sum(a1.to(dev), b1[0].contiguous().to(dev), a2.to(dev), b2[0].contiguous().to(dev))
+    assert_grad_close(dense, a1.double() @ b1[0].double().t() + a2.double() @ b2[0].double().t(), "bf16", "dense")
+
+
 @pytest.mark.parametrize("rows,d,f", [([5, 0, 300, 64, 1, 700], 128, 192), ([130, 257], 64, 64), ([0, 0, 9], 256, 128)])
 def test_grouped_swiglu_keep_leaves_the_two_products(gpu_device, rows, d, f):
     """The training-forward variant of the expert kernel: same ``ye`` and ``h`` as the inference
