@@ -56,6 +56,7 @@ _PROTOTYPES = {
     ),
     "fs2moe_grouped_swiglu_fuses_gather": (c_int32, [c_int32, c_int32, c_int32, c_int32]),
     "fs2moe_grouped_swiglu_keeps": (c_int32, [c_int32, c_int32, c_int64, c_int32]),
+    "fs2moe_dense_swiglu_keep": (c_int32, [c_void_p] * 4 + [c_int32] * 4 + [c_void_p] * 5),
     "fs2moe_grouped_gemm_sum_supported": (c_int32, [c_int32, c_int32, c_int64, c_int32]),
     "fs2moe_grouped_gemm_sum": (
         c_int32, [c_void_p] * 6 + [c_int32] * 3 + [c_int64, c_int32, c_void_p, c_void_p],
@@ -468,6 +469,25 @@ def dense_swiglu(x: Tensor, w_gate: Tensor, w_up: Tensor, w_down: Tensor) -> Ten
     )
     _check(rc, "fs2moe_dense_swiglu")
     return y
+
+
+def dense_swiglu_keep(x: Tensor, w_gate: Tensor, w_up: Tensor, w_down: Tensor) -> tuple[Tensor, Tensor, Tensor]:
+    """:func:`dense_swiglu` that also returns the gate and the up product: ``(y, g, u)``."""
+    lib = load()
+    t, d = x.shape
+    f = w_gate.shape[0]
+    if w_gate.shape != (f, d) or w_up.shape != (f, d) or w_down.shape != (d, f):
+        raise ValueError("shared-expert weights must be (F, D), (F, D), (D, F)")
+    for name, w in (("w_gate", w_gate), ("w_up", w_up), ("w_down", w_down)):
+        _same(name, w, w.shape, x.dtype, x.device)
+    g, u, h = (torch.empty((t, f), dtype=x.dtype, device=x.device) for _ in range(3))
+    y = torch.empty((t, d), dtype=x.dtype, device=x.device)
+    rc = lib.fs2moe_dense_swiglu_keep(
+        _ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(w_down), t, d, f, dtype_code(x.dtype), _ptr(g),
+        _ptr(u), _ptr(h), _ptr(y), _stream(),
+    )
+    _check(rc, "fs2moe_dense_swiglu_keep")
+    return y, g, u
 
 
 def combine(

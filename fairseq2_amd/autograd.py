@@ -46,15 +46,20 @@ def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg):
         ye, _, g, u = _abi.grouped_swiglu_keep(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
     else:
         ye, _ = _abi.grouped_swiglu(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
-    base = _abi.dense_swiglu(x, sg, su, sd) if sg is not None else None
+    base = g_s = u_s = None
+    if sg is not None:
+        if _abi.keeps_products(x.shape[1], sg.shape[0], x.shape[0], x.dtype):
+            base, g_s, u_s = _abi.dense_swiglu_keep(x, sg, su, sd)
+        else:
+            base = _abi.dense_swiglu(x, sg, su, sd)
     out = _abi.combine(ye, disp.inv_perm, idx, w, base, not scale_input, out=base, residual=residual)
-    return out, (idx, w, logits, disp.counts, disp.offsets, disp.inv_perm, disp.xe, ye, g, u)
+    return out, (idx, w, logits, disp.counts, disp.offsets, disp.inv_perm, disp.xe, ye, g, u, g_s, u_s)
 
 
 def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
     """Gradients ``(dx, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd)`` (None where ``need`` -- in
     that order -- says so) from the output gradient and the intermediates of :func:`forward_saving`."""
-    idx, w, logits, counts, offsets, inv_perm, xe, ye, g, u = saved
+    idx, w, logits, counts, offsets, inv_perm, xe, ye, g, u, g_s, u_s = saved
     e, tile_m = cfg["num_experts"], cfg["tile_m"]
     score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
     dout = dout.contiguous()
@@ -94,9 +99,12 @@ def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
     d_sg = d_su = d_sd = None
     if sg is not None:
         dh_s = _abi.grouped_gemm(dout, sd, IN_OUT)
-        g_s = _abi.grouped_gemm(x, sg, OUT_IN)
-        u_s = _abi.grouped_gemm(x, su, OUT_IN)
-        h_s, dg_s, du_s = _abi.swiglu_backward(g_s, u_s, dh_s)
+        if g_s is None:
+            g_s = _abi.grouped_gemm(x, sg, OUT_IN)
+            u_s = _abi.grouped_gemm(x, su, OUT_IN)
+            h_s, dg_s, du_s = _abi.swiglu_backward(g_s, u_s, dh_s)
+        else:
+            h_s, dg_s, du_s = _abi.swiglu_backward(g_s, u_s, dh_s, in_place=False)
         d_sd = _abi.grouped_wgrad(dout, h_s) if need[7] else None
         d_sg = _abi.grouped_wgrad(dg_s, x) if need[5] else None
         d_su = _abi.grouped_wgrad(du_s, x) if need[6] else None

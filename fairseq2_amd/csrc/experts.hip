@@ -338,12 +338,12 @@ static int launch_dma_pair(const void* x, const int32_t* row_map, const Groups& 
   using namespace dma;
   const int groups = g.counts ? g.E : 0;
   // the gate/up kernel, or its variant that also stores the two products (plain bf16 weights only)
-  constexpr bool CAN_KEEP = BLAYOUT == FS2MOE_W_IN_OUT;
+  constexpr bool CAN_KEEP = BLAYOUT != dma::W_FP8_TILED;
   auto k1 = glu_gemm_bf16_dma_kernel<true, BLAYOUT>;
   auto k1k = glu_gemm_bf16_dma_kernel<true, BLAYOUT, CAN_KEEP>;
   auto k2 = glu_gemm_bf16_dma_kernel<false, BLAYOUT>;
   if (g_keep != nullptr && !CAN_KEEP) {
-    set_error("experts: the products are kept with bf16 weights in the (in, out) layout only");
+    set_error("experts: the products are kept with bf16 weights only");
     return FS2MOE_ERR_UNSUPPORTED;
   }
   static bool attr_set = false;  // benign race: setting the attribute is idempotent
@@ -676,6 +676,27 @@ extern "C" int fs2moe_grouped_gemm(const void* a, const int32_t* row_map, const 
   if (b_layout == FS2MOE_W_IN_OUT)
     return launch_gemm<FS2MOE_W_IN_OUT>(a, row_map, g, max_rows, b, K, N, dtype, c, st);
   return launch_gemm<FS2MOE_W_OUT_IN>(a, row_map, g, max_rows, b, K, N, dtype, c, st);
+}
+
+extern "C" int fs2moe_dense_swiglu_keep(const void* x, const void* w_gate, const void* w_up,
+                                        const void* w_down, int32_t T, int32_t D, int32_t F,
+                                        int32_t act_dtype, void* g, void* u, void* h, void* y,
+                                        void* stream) {
+  FS2_REQUIRE(x && w_gate && w_up && w_down && g && u && h && y, "dense_swiglu_keep: null pointer");
+  FS2_REQUIRE(T >= 0, "dense_swiglu_keep: T=%d", T);
+  if (!fs2moe_grouped_swiglu_keeps(D, F, T, act_dtype)) {
+    set_error("dense_swiglu_keep: needs bf16, D and F multiples of 64 and activation matrices "
+              "below 4 GB (D=%d, F=%d, act_dtype %d, T=%d)", D, F, act_dtype, T);
+    return FS2MOE_ERR_UNSUPPORTED;
+  }
+  FS2_REQUIRE(aligned16(x) && aligned16(w_gate) && aligned16(w_up) && aligned16(w_down) &&
+                  aligned16(g) && aligned16(u) && aligned16(h) && aligned16(y),
+              "dense_swiglu_keep: buffers must be 16-byte aligned");
+  if (T == 0) return FS2MOE_OK;
+  Groups grp{nullptr, nullptr, 1, T};
+  return launch_dma_pair<FS2MOE_W_OUT_IN>(x, nullptr, grp, T, w_gate, w_up, w_down, nullptr,
+                                          nullptr, nullptr, D, F, h, y,
+                                          static_cast<hipStream_t>(stream), g, u);
 }
 
 extern "C" int fs2moe_grouped_gemm_sum_supported(int32_t K, int32_t N, int64_t max_rows,

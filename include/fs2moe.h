@@ -305,6 +305,10 @@ int fs2moe_grouped_gemm_sum(const void* a1, const void* b1, const void* a2, cons
  *   g, u [max_rows, F] (out); everything else as for fs2moe_grouped_swiglu.
  */
 int fs2moe_grouped_swiglu_keeps(int32_t D, int32_t F, int64_t max_rows, int32_t act_dtype);
+/* The same for the shared expert (fs2moe_dense_swiglu; max_rows = T in fs2moe_grouped_swiglu_keeps). */
+int fs2moe_dense_swiglu_keep(const void* x, const void* w_gate, const void* w_up,
+                             const void* w_down, int32_t T, int32_t D, int32_t F, int32_t act_dtype,
+                             void* g, void* u, void* h, void* y, void* stream);
 int fs2moe_grouped_swiglu_keep(const void* xe, const int32_t* row_map, const int32_t* counts,
                                const int32_t* offsets, const void* w_gate, const void* w_up,
                                const void* w_down, int32_t E, int32_t D, int32_t F,

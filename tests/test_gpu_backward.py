@@ -194,6 +194,23 @@ def test_full_size_weight_gradient_and_kept_products(gpu_device):
         assert_grad_close(up[sl], ref.double().cpu(), "bf16", f"up product of expert {ex}")
 
 
+def test_dense_swiglu_keep_leaves_the_two_products(gpu_device):
+    """The shared expert's training forward: ``y`` as the inference kernel gives it, bit for bit, and
+    the two products as two GEMMs give them."""
+    dev = gpu_device
+    g = torch.Generator().manual_seed(3)
+    t, d, f = 300, 128, 192
+    x = torch.randn(t, d, generator=g).to(torch.bfloat16).to(dev)
+    wg, wu = ((0.2 * torch.randn(f, d, generator=g)).to(torch.bfloat16).to(dev) for _ in range(2))
+    wd = (0.2 * torch.randn(d, f, generator=g)).to(torch.bfloat16).to(dev)
+    y0 = _abi.dense_swiglu(x, wg, wu, wd)
+    y, gate, up = _abi.dense_swiglu_keep(x, wg, wu, wd)
+    assert torch.equal(y, y0)
+    assert torch.equal(gate, _abi.grouped_gemm(x, wg, _abi.W_OUT_IN))
+    assert torch.equal(up, _abi.grouped_gemm(x, wu, _abi.W_OUT_IN))
+    assert_grad_close(gate, x.double().cpu() @ wg.double().cpu().t(), "bf16", "gate product")
+
+
 def test_backward_twice_gives_the_same_gradients(gpu_device):
     """The kept products are autograd's saved tensors: a backward pass must leave them as they are
     (``retain_graph=True`` and a second pass is how a trainer accumulates two losses)."""
