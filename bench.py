@@ -31,12 +31,12 @@ MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3, "fp8": 5000.0}  # dense, publ
 MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     # profiles/bench_<workload>_all_kernels.md, the two launches of fs2moe_grouped_swiglu together
     # (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0 against a 256 MiB copy)
-    "qwen3_30b_a3b": 2.643e9,     # gate/up 1542 + 101 MB, down 730 + 271 MB
-    "mixtral_8x7b": 15.091e9,     # gate/up 10404 + 470 MB, down 4081 + 136 MB
-    "llama4_scout": 6.632e9,      # routed experts only: gate/up 4234 + 134 MB, down 2178 + 86 MB
+    "qwen3_30b_a3b": 2.650e9,     # gate/up 1549 + 101 MB, down 729 + 270 MB
+    "mixtral_8x7b": 14.950e9,     # gate/up 10286 + 470 MB, down 4058 + 136 MB
+    "llama4_scout": 6.639e9,      # routed experts only: gate/up 4231 + 134 MB, down 2188 + 86 MB
     "small_fp32": 0.862e9,        # gate/up 398 + 46 MB, down 401 + 17 MB
     "qwen3_decode_fp8": 0.224e9,  # gate/up 142 + 1 MB, down 77 + 4 MB
-    "qwen3_30b_a3b_fp8": 1.896e9,  # gate/up 1035 + 101 MB, down 491 + 270 MB
+    "qwen3_30b_a3b_fp8": 1.895e9,  # gate/up 1035 + 101 MB, down 490 + 270 MB
 }
 
 
