@@ -42,7 +42,16 @@ def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg):
     # where the expert kernel can, it leaves the gate and the up product behind for the backward
     # pass (what autograd would save); otherwise backward_from computes them again
     g = u = None
-    if _abi.keeps_products(x.shape[1], wd.shape[0] // e, disp.xe.shape[0], x.dtype):
+    act = cfg.get("activation")
+    if act is not None:
+        # a gate activation other than SiLU (experts.py:84-87 takes any module): the module's own
+        # forward between the library's plain grouped GEMMs, in f32 with one rounding
+        grp = dict(counts=disp.counts, offsets=disp.offsets, num_experts=e)
+        g = _abi.grouped_gemm(disp.xe, wg, _abi.W_IN_OUT, **grp)
+        u = _abi.grouped_gemm(disp.xe, wu, _abi.W_IN_OUT, **grp)
+        h = (act(g.float()) * u.float()).to(x.dtype)
+        ye = _abi.grouped_gemm(h, wd, _abi.W_IN_OUT, **grp)
+    elif _abi.keeps_products(x.shape[1], wd.shape[0] // e, disp.xe.shape[0], x.dtype):
         ye, _, g, u = _abi.grouped_swiglu_keep(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
     else:
         ye, _ = _abi.grouped_swiglu(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
@@ -70,7 +79,17 @@ def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
     # the permutation is the forward pass's: dispatch is deterministic
     dye = _abi.dispatch(idx, w, dout, e, tile_m, not scale_input, gather=True).xe
     dh = _abi.grouped_gemm(dye, wd, OUT_IN, **grp)
-    if g is None:
+    act = cfg.get("activation")
+    if act is not None:
+        # the module's own derivative, through torch.autograd on its forward (f32, one rounding)
+        with torch.enable_grad():
+            g32 = g.float().requires_grad_(True)
+            a32 = act(g32)
+        u32, dh32 = u.float(), dh.float()
+        (dg32,) = torch.autograd.grad(a32, g32, dh32 * u32)
+        a32 = a32.detach()
+        h, dg, du = (a32 * u32).to(x.dtype), dg32.to(x.dtype), (dh32 * a32).to(x.dtype)
+    elif g is None:
         g = _abi.grouped_gemm(xe, wg, IN_OUT, **grp)
         u = _abi.grouped_gemm(xe, wu, IN_OUT, **grp)
         h, dg, du = _abi.swiglu_backward(g, u, dh)  # in place over g and u

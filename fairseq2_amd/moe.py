@@ -210,8 +210,10 @@ class GroupedExpertNetwork(ExpertNetwork):
             if self.has_fp8_weights or row_map is not None:
                 raise NotImplementedError("e4m3 weights and the fused gather need the SiLU gate")
             grp = dict(counts=counts, offsets=offsets, num_experts=self.num_local_experts)
-            h = self.activation(_abi.grouped_gemm(xe, self.gate_proj.detach(), _abi.W_IN_OUT, **grp))
-            h = (h * _abi.grouped_gemm(xe, self.inner_proj.detach(), _abi.W_IN_OUT, **grp)).to(xe.dtype)
+            # (in f32 with one rounding, like the fused SiLU gate; the training path does the same)
+            g = _abi.grouped_gemm(xe, self.gate_proj.detach(), _abi.W_IN_OUT, **grp)
+            u = _abi.grouped_gemm(xe, self.inner_proj.detach(), _abi.W_IN_OUT, **grp)
+            h = (self.activation(g.float()) * u.float()).to(xe.dtype)
             return _abi.grouped_gemm(h.contiguous(), self.output_proj.detach(), _abi.W_IN_OUT, **grp)
         if self.has_fp8_weights:
             ye, _ = _abi.grouped_swiglu(
@@ -461,8 +463,8 @@ class MoE(FeedForwardNetwork):
             why = "the normalisation fused into the router has no backward pass (normalise outside the layer)"
         elif type(ex) is not GroupedExpertNetwork or (se is not None and type(se) is not GLUFeedForwardNetwork):
             why = "only GroupedExpertNetwork experts and a GLUFeedForwardNetwork shared expert are differentiated"
-        elif not ex.has_fused_gate:
-            why = "only the SiLU gate is differentiated"
+        elif not ex.has_fused_gate and any(p.requires_grad for p in ex.activation.parameters()):
+            why = "a gate activation with parameters of its own is not differentiated"
         elif ex.has_fp8_weights:
             why = "e4m3 expert weights are an inference format"
         elif ex.num_local_experts % 8:
@@ -494,6 +496,7 @@ class MoE(FeedForwardNetwork):
             num_experts=ex.num_local_experts, top_k=self.top_k, tile_m=self.tile_m,
             score_fn=_SCORE_FNS[self.score_fn], renormalize=self.renormalize,
             scale_input=self.scale_on == "input", router_bias=self.router_bias,
+            activation=None if ex.has_fused_gate else ex.activation,
         )
         out = MoEFunction.apply(x, res, self.router, ex.gate_proj, ex.inner_proj, ex.output_proj,
                                 *shared, cfg)

@@ -216,8 +216,10 @@ def ref_dense_forward(
     score_fn: str = "sigmoid",
     renormalize: bool = False,
     scale_on: str = "input",
+    activation=F.silu,
 ) -> Tensor:
-    """The reference's dense formulation, op for op (``moe.py:102-157``).
+    """The reference's dense formulation, op for op (``moe.py:102-157``).  ``activation`` is the
+    routed experts' gate activation (``experts.py:84-87``: any module, SiLU by default).
 
     Every expert runs over all T tokens; unselected pairs get a zero input
     (reference mode) or a zero weight (output-weighted extension).
@@ -253,7 +255,7 @@ def ref_dense_forward(
     wg = gate.view(num_experts, -1, gate.shape[-1])
     wu = up.view(num_experts, -1, up.shape[-1])
     wd = down.view(num_experts, -1, down.shape[-1])
-    h = F.silu(torch.bmm(routed_input, wg))
+    h = activation(torch.bmm(routed_input, wg))
     h = h * torch.bmm(routed_input, wu)
     routed_output = torch.bmm(h, wd).reshape(-1, dim)
     if scale_on == "output":

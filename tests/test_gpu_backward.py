@@ -321,7 +321,7 @@ MODES = {
 }
 
 
-def _reference_gradients(wl, grad_out, residual):
+def _reference_gradients(wl, grad_out, residual, activation=None):
     """float64 autograd through the dense restatement of the reference layer."""
     s = wl.spec
     c = lambda t: None if t is None else t.double().clone().requires_grad_(True)  # noqa: E731
@@ -332,6 +332,7 @@ def _reference_gradients(wl, grad_out, residual):
         x, router, gate, up, down, s.top_k, shared=shared,
         router_bias=None if wl.router_bias is None else wl.router_bias.double(),
         score_fn=s.mode.score_fn, renormalize=s.mode.renormalize, scale_on=s.mode.scale_on,
+        **({} if activation is None else {"activation": activation}),
     )
     if res is not None:
         out = out + res
@@ -387,6 +388,30 @@ def test_layer_gradients_match_autograd_of_the_reference(gpu_device, dtype, mode
         assert_grad_close(p.grad, ref[name], dtype, f"d {name}")
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("mode,shared", [("reference", True), ("softmax_renorm_output", False)])
+def test_gradients_with_another_gate_activation(gpu_device, dtype, mode, shared):
+    """``moe_activation`` other than SiLU (``llama4/moe.py:44``, ``experts.py:84-87`` take any
+    module): the module's own derivative between the library's GEMMs, against float64 autograd
+    through the same dense restatement with that activation."""
+    act = torch.nn.GELU(approximate="tanh")
+    spec = W.small_spec(tokens=257, model_dim=128, num_experts=16, top_k=2, inner_dim=192, dtype=dtype,
+                        shared=shared, zipf_s=1.0, mode=MODES[mode], seed=21)
+    wl = W.make_workload_from_spec(spec)
+    dt = TORCH_DTYPE[dtype]
+    g = torch.Generator().manual_seed(5)
+    grad_out = torch.randn(wl.x.shape, generator=g).to(dt).float()
+    _, ref = _reference_gradients(wl, grad_out, None, activation=act)
+    m = build_module(wl, gpu_device)
+    m.experts.activation = act
+    m.train().requires_grad_(True)
+    x = wl.x.to(dt).to(gpu_device).requires_grad_(True)
+    m(x).backward(grad_out.to(dt).to(gpu_device))
+    assert_grad_close(x.grad, ref["x"], dtype, "d x")
+    for name, p in m.named_parameters():
+        assert_grad_close(p.grad, ref[name], dtype, f"d {name}")
+
+
 def test_frozen_parameters_get_no_gradient_and_unsupported_cases_say_so(gpu_device):
     wl = W.make_workload_from_spec(W.small_spec(dtype="bf16", tokens=64, num_experts=8, inner_dim=128, seed=3))
     m = build_module(wl, gpu_device)  # frozen
@@ -400,6 +425,10 @@ def test_frozen_parameters_get_no_gradient_and_unsupported_cases_say_so(gpu_devi
 
     with pytest.raises(RuntimeError, match="no backward pass"):
         m(x, norm=_Norm)
+    m.experts.activation = torch.nn.PReLU().to(gpu_device)
+    with pytest.raises(RuntimeError, match="parameters of its own"):
+        m(x)
+    m.experts.activation = torch.nn.SiLU()
     m.experts.quantize_fp8_()
     with pytest.raises(RuntimeError, match="inference format"):
         m(x)
