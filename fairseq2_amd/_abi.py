@@ -185,6 +185,27 @@ def _ptr(t: Tensor | None) -> int | None:
     return t.data_ptr()
 
 
+def _same(name: str, t: Tensor, shape: tuple, dtype: torch.dtype, dev: torch.device) -> None:
+    if tuple(t.shape) != tuple(shape) or t.dtype != dtype or t.device != dev or not t.is_contiguous():
+        raise ValueError(
+            f"{name} must be a contiguous {tuple(shape)} {dtype} tensor on {dev}, got {tuple(t.shape)} "
+            f"{t.dtype} on {t.device}")
+
+
+def _check_groups(counts: Tensor, offsets: Tensor, num_experts: int, dev: torch.device) -> None:
+    _same("counts", counts, (num_experts,), torch.int32, dev)
+    _same("offsets", offsets, (num_experts + 1,), torch.int32, dev)
+
+
+def _check_selection(topk_idx: Tensor, topk_w: Tensor | None, dev: torch.device) -> tuple[int, int]:
+    if topk_idx.dim() != 2:
+        raise ValueError("topk_idx must be (T, K)")
+    _same("topk_idx", topk_idx, topk_idx.shape, torch.int32, dev)
+    if topk_w is not None:
+        _same("topk_w", topk_w, topk_idx.shape, torch.float32, dev)
+    return topk_idx.shape[0], topk_idx.shape[1]
+
+
 def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
@@ -310,9 +331,13 @@ def dispatch(
     gather: bool = True,
 ) -> Dispatched:
     lib = load()
-    t, k = topk_idx.shape
-    d = x.shape[1]
     dev = x.device
+    t, k = _check_selection(topk_idx, topk_w, dev)
+    if x.dim() != 2 or x.shape[0] != t:
+        raise ValueError("x must be (T, D) with one row per row of topk_idx")
+    if scale_input and topk_w is None:
+        raise ValueError("scaling the rows needs topk_w")
+    d = x.shape[1]
     rows = max_rows(t, k, num_experts, tile_m)
     counts = torch.empty(num_experts, dtype=torch.int32, device=dev)
     offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
@@ -380,12 +405,15 @@ def grouped_swiglu(
         if row_map.dtype != torch.int32 or row_map.dim() != 1:
             raise ValueError("row_map must be a 1-d int32 tensor")
         rows = row_map.shape[0]
+    _check_groups(counts, offsets, num_experts, xe.device)
     if scales is None:
         f = w_down.shape[0] // num_experts
         if w_gate.shape != (num_experts * d, f) or w_up.shape != w_gate.shape:
             raise ValueError("gate/up weights must be (E*D, F)")
         if w_down.shape != (num_experts * f, d):
             raise ValueError("down weights must be (E*F, D)")
+        for name, w in (("w_gate", w_gate), ("w_up", w_up), ("w_down", w_down)):
+            _same(name, w, w.shape, xe.dtype, xe.device)
     else:
         f = w_gate.shape[1] * 16
         if w_gate.shape != (num_experts, f // 16, d // 64, 16, 64) or w_up.shape != w_gate.shape:
@@ -395,6 +423,9 @@ def grouped_swiglu(
         want = [(num_experts, f), (num_experts, f), (num_experts, d)]
         if [tuple(s.shape) for s in scales] != want or any(s.dtype != torch.float32 for s in scales):
             raise ValueError("fp8 scales must be f32 (E, F), (E, F), (E, D)")
+        for w in (w_gate, w_up, w_down):
+            if w.dtype not in (torch.float8_e4m3fn, torch.uint8) or w.device != xe.device:
+                raise ValueError("fp8 codes must be float8_e4m3fn (or their uint8 bytes) on the device of xe")
     h = torch.empty((rows, f), dtype=xe.dtype, device=xe.device)
     ye = torch.empty((rows, d), dtype=xe.dtype, device=xe.device)
     sg, su, sd = scales if scales is not None else (None, None, None)
@@ -426,7 +457,10 @@ def grouped_swiglu_keep(
     lib = load()
     rows, d = xe.shape
     if row_map is not None:
+        if row_map.dtype != torch.int32 or row_map.dim() != 1:
+            raise ValueError("row_map must be a 1-d int32 tensor")
         rows = row_map.shape[0]
+    _check_groups(counts, offsets, num_experts, xe.device)
     f = w_down.shape[0] // num_experts
     if w_gate.shape != (num_experts * d, f) or w_up.shape != w_gate.shape:
         raise ValueError("gate/up weights must be (E*D, F)")
@@ -461,6 +495,8 @@ def dense_swiglu(x: Tensor, w_gate: Tensor, w_up: Tensor, w_down: Tensor) -> Ten
     f = w_gate.shape[0]
     if w_gate.shape != (f, d) or w_up.shape != (f, d) or w_down.shape != (d, f):
         raise ValueError("shared-expert weights must be (F, D), (F, D), (D, F)")
+    for name, w in (("w_gate", w_gate), ("w_up", w_up), ("w_down", w_down)):
+        _same(name, w, w.shape, x.dtype, x.device)
     h = torch.empty((t, f), dtype=x.dtype, device=x.device)
     y = torch.empty((t, d), dtype=x.dtype, device=x.device)
     rc = lib.fs2moe_dense_swiglu(
@@ -503,10 +539,17 @@ def combine(
     """``out[t] = (residual[t] +) base[t] + sum of the token's expert rows``; ``out`` may be
     ``base`` or ``residual`` itself."""
     lib = load()
-    t, k = inv_perm.shape
+    t, k = _check_selection(topk_idx, topk_w, ye.device)
+    _same("inv_perm", inv_perm, (t, k), torch.int32, ye.device)
+    if weight_output and topk_w is None:
+        raise ValueError("weighting the output needs topk_w")
     d = ye.shape[1]
+    if base is not None:
+        _same("base", base, (t, d), ye.dtype, ye.device)
     if out is None:
         out = torch.empty((t, d), dtype=ye.dtype, device=ye.device)
+    else:
+        _same("out", out, (t, d), ye.dtype, ye.device)
     if residual is None:
         rc = lib.fs2moe_combine(
             _ptr(ye), _ptr(inv_perm), _ptr(topk_idx), _ptr(topk_w), _ptr(base), t, k, d,
@@ -514,8 +557,7 @@ def combine(
         )
         _check(rc, "fs2moe_combine")
     else:
-        if residual.shape != (t, d) or residual.dtype != ye.dtype or not residual.is_contiguous():
-            raise ValueError("residual must be a contiguous (T, D) tensor of the activation dtype")
+        _same("residual", residual, (t, d), ye.dtype, ye.device)
         rc = lib.fs2moe_combine_residual(
             _ptr(ye), _ptr(inv_perm), _ptr(topk_idx), _ptr(topk_w), _ptr(base), _ptr(residual), t, k,
             d, dtype_code(ye.dtype), int(weight_output), _ptr(out), _stream(),
@@ -525,13 +567,6 @@ def combine(
 
 
 # ---------------------------------------------------------------------------------- backward pass
-def _same(name: str, t: Tensor, shape: tuple, dtype: torch.dtype, dev: torch.device) -> None:
-    if tuple(t.shape) != tuple(shape) or t.dtype != dtype or t.device != dev or not t.is_contiguous():
-        raise ValueError(
-            f"{name} must be a contiguous {tuple(shape)} {dtype} tensor on {dev}, got {tuple(t.shape)} "
-            f"{t.dtype} on {t.device}")
-
-
 def grouped_gemm(
     a: Tensor,
     b: Tensor,

@@ -112,7 +112,13 @@ def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
     else:
         d_w = _abi.pair_dot(ye, inv_perm, dout)
     dl = _abi.router_backward(logits, idx, w, d_w, score_fn, renorm, x.dtype)
-    d_router = _abi.grouped_wgrad(x, dl) if need[1] else None
+    # the two products with the router matrix read rows of 16 bytes: with a number of experts that
+    # is not a multiple of 8, zero columns are appended (they add nothing) and cut off again
+    pad = -e % 8
+    if pad:
+        dl = torch.nn.functional.pad(dl, (0, pad))
+        router = torch.nn.functional.pad(router, (0, pad))
+    d_router = _abi.grouped_wgrad(x, dl)[:, :e].contiguous() if need[1] else None
     dx_parts = [_abi.grouped_gemm(dl, router, OUT_IN)] if need[0] else []
 
     d_sg = d_su = d_sd = None

@@ -450,6 +450,11 @@ class MoE(FeedForwardNetwork):
         if (type(ex) is GroupedExpertNetwork and ex.has_fused_gate
                 and (se is None or type(se) is GLUFeedForwardNetwork)):
             return self._single_call(x, res, norm_args).view(seqs.shape)
+        if wants_grad:
+            # (only reachable inside a compiler's trace: the staged path below records no graph)
+            raise RuntimeError(
+                "fairseq2_amd.MoE: under torch.compile only the fused SiLU experts are differentiated; "
+                "train this configuration eagerly")
         return self._stages(x, res, norm_args)[0].view(seqs.shape)
 
     def _differentiable(self, seqs: Tensor, residual: Tensor | None, norm) -> Tensor:
@@ -467,8 +472,6 @@ class MoE(FeedForwardNetwork):
             why = "a gate activation with parameters of its own is not differentiated"
         elif ex.has_fp8_weights:
             why = "e4m3 expert weights are an inference format"
-        elif ex.num_local_experts % 8:
-            why = "the router's backward kernels need a number of experts that is a multiple of 8"
         if why is not None:
             raise RuntimeError(
                 f"fairseq2_amd.MoE: {why}; call it under torch.no_grad() / torch.inference_mode(), "

@@ -113,9 +113,6 @@ def _setup_context(ctx, inputs, output):
     if s_gate is not None or normed:
         ctx.unsupported = "e4m3 weights and the fused normalisation are forward-only"
         return
-    if num_experts % 8:
-        ctx.unsupported = "the router's backward kernels need a number of experts that is a multiple of 8"
-        return
     ctx.unsupported = None
     ctx.ints = (num_experts, top_k, tile_m, score_fn, renormalize, scale_input)
     ctx.has_residual = residual is not None

@@ -208,6 +208,61 @@ def test_extension_options_are_validated():
     assert "router_bias" in m.state_dict()
 
 
+def test_stage_wrappers_check_their_tensors_before_calling_the_library():
+    """A tensor of the wrong shape or type must raise on the host: the library takes raw pointers
+    and would read it as what it expects.  (Host tensors: every check below fails before a pointer
+    is taken.)"""
+    e, d, f, t, k = 4, 64, 64, 6, 2
+    bf = torch.bfloat16
+    xe = torch.zeros(16, d, dtype=bf)
+    counts, offsets = torch.zeros(e, dtype=torch.int32), torch.zeros(e + 1, dtype=torch.int32)
+    wg, wu, wd = torch.zeros(e * d, f, dtype=bf), torch.zeros(e * d, f, dtype=bf), torch.zeros(e * f, d, dtype=bf)
+    idx, w = torch.zeros(t, k, dtype=torch.int32), torch.zeros(t, k)
+    inv = torch.zeros(t, k, dtype=torch.int32)
+    for fn in (_abi.grouped_swiglu, _abi.grouped_swiglu_keep):
+        with pytest.raises(ValueError, match="counts"):
+            fn(xe, counts.long(), offsets, wg, wu, wd, e)
+        with pytest.raises(ValueError, match="offsets"):
+            fn(xe, counts, offsets[:-1], wg, wu, wd, e)
+        with pytest.raises(ValueError, match="w_up"):
+            fn(xe, counts, offsets, wg, wu.float(), wd, e)
+        with pytest.raises(ValueError, match="down weights"):
+            fn(xe, counts, offsets, wg, wu, torch.zeros(e * f, d + 8, dtype=bf), e)
+        with pytest.raises(ValueError, match="row_map"):
+            fn(xe, counts, offsets, wg, wu, wd, e, row_map=torch.zeros(16, dtype=torch.int64))
+    for fn in (_abi.dense_swiglu, _abi.dense_swiglu_keep):
+        with pytest.raises(ValueError, match="w_gate"):
+            fn(xe, torch.zeros(f, d), torch.zeros(f, d, dtype=bf), torch.zeros(d, f, dtype=bf))
+        with pytest.raises(ValueError, match="shared-expert weights"):
+            fn(xe, torch.zeros(f, d, dtype=bf), torch.zeros(f, d, dtype=bf), torch.zeros(d, f + 8, dtype=bf))
+    x = torch.zeros(t, d, dtype=bf)
+    with pytest.raises(ValueError, match="topk_idx"):
+        _abi.dispatch(idx.long(), w, x, e, 1, False)
+    with pytest.raises(ValueError, match="topk_w"):
+        _abi.dispatch(idx, w.double(), x, e, 1, False)
+    with pytest.raises(ValueError, match="one row per row"):
+        _abi.dispatch(idx, w, x[:-1], e, 1, False)
+    with pytest.raises(ValueError, match="needs topk_w"):
+        _abi.dispatch(idx, None, x, e, 1, True)
+    ye = torch.zeros(t * k, d, dtype=bf)
+    with pytest.raises(ValueError, match="inv_perm"):
+        _abi.combine(ye, inv[:, :1], idx, w, None, True)
+    with pytest.raises(ValueError, match="base"):
+        _abi.combine(ye, inv, idx, w, x.float(), True)
+    with pytest.raises(ValueError, match="out"):
+        _abi.combine(ye, inv, idx, w, None, True, out=torch.zeros(t, d + 8, dtype=bf))
+    with pytest.raises(ValueError, match="residual"):
+        _abi.combine(ye, inv, idx, w, None, True, residual=x[:-1])
+    with pytest.raises(ValueError, match="needs topk_w"):
+        _abi.combine(ye, inv, idx, None, None, True)
+    with pytest.raises(ValueError, match="a2"):
+        _abi.grouped_gemm_sum(xe, wg.view(e * f, d), xe.float(), wg.view(e * f, d), counts, offsets, e)
+    with pytest.raises(ValueError, match="same number of rows"):
+        _abi.grouped_wgrad(xe, xe[:-1].contiguous(), counts, offsets, e)
+    with pytest.raises(ValueError, match="dh"):
+        _abi.swiglu_backward(xe, xe.clone(), xe.float())
+
+
 def test_no_cpu_fallback_and_forward_only():
     m = M.MoE(64, 64, False, 4, 1.0, 1, inner_dim_scale=1.0, auto_scale=False)
     x = torch.zeros(2, 3, 64)
