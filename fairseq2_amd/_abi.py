@@ -15,7 +15,7 @@ from torch import Tensor
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfs2moe.so")
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
@@ -120,6 +120,12 @@ _PROTOTYPES = {
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32,
          c_int32, c_void_p, c_void_p],
+    ),
+    "fs2moe_rms_norm_backward_workspace_bytes": (c_int64, [c_int32, c_int32]),
+    "fs2moe_rms_norm_backward": (
+        c_int32,
+        [c_void_p, c_void_p, c_float, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p,
+         c_void_p, c_int64, c_void_p],
     ),
     "fs2moe_forward_norm": (
         c_int32,
@@ -743,6 +749,31 @@ def router_backward(logits: Tensor, topk_idx: Tensor, topk_w: Tensor, d_w: Tenso
                                     score_fn, int(renormalize), dtype_code(dtype), _ptr(dl), _stream())
     _check(rc, "fs2moe_router_backward")
     return dl
+
+
+def rms_norm_backward(x: Tensor, weight: Tensor | None, eps: float, dy: Tensor,
+                      want_weight_grad: bool = True) -> tuple[Tensor, Tensor | None]:
+    """``(dx, dweight)`` of ``y = rms_norm(x) * weight`` given ``dy`` (``fs2moe_rms_norm_backward``);
+    ``dweight`` is None without a weight or when not asked for."""
+    lib = load()
+    t, d = x.shape
+    _same("x", x, (t, d), x.dtype, x.device)
+    _same("dy", dy, (t, d), x.dtype, x.device)
+    if weight is not None:
+        _same("weight", weight, (d,), x.dtype, x.device)
+    dx = torch.empty_like(x)
+    dw = ws = None
+    ws_bytes = 0
+    if weight is not None and want_weight_grad:
+        dw = torch.empty_like(weight)
+        ws_bytes = lib.fs2moe_rms_norm_backward_workspace_bytes(t, d)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    rc = lib.fs2moe_rms_norm_backward(
+        _ptr(x), _ptr(weight), float(eps), _ptr(dy), t, d, dtype_code(x.dtype), _ptr(dx), _ptr(dw),
+        _ptr(ws), ws_bytes, _stream(),
+    )
+    _check(rc, "fs2moe_rms_norm_backward")
+    return dx, dw
 
 
 def check_layer_arguments(x, router, router_bias, w_gate, w_up, w_down, num_experts, f, scales, shared) -> None:

@@ -21,6 +21,10 @@ derivation is written out once, against ``moe.py:102-157``, ``experts.py:102-112
     drouter  = x^T dlogits,  dx += dlogits @ router^T                          -> wgrad / gemm, one group
     dx      += sum_k s_k * dxe[row]            scattered back to token order   -> fs2moe_combine
 
+With the layer's RMS normalisation in front (``decoder_layer.py:187-191``) ``x`` above is the
+normalised rows ``xn`` that the router kernel wrote, and one more step turns their gradient into
+that of the raw rows and of the norm's weight                                  -> fs2moe_rms_norm_backward
+
 The discrete selection (``torch.topk``) has no gradient, as in the reference.  Intermediates are
 rounded to the activation dtype between kernels, as autograd's would be.
 """
@@ -33,11 +37,17 @@ from torch import Tensor
 from fairseq2_amd import _abi
 
 
-def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg):
-    """The staged forward pass; returns ``(out, saved)`` with what :func:`backward_from` needs."""
+def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg, norm_w=None):
+    """The staged forward pass; returns ``(out, saved)`` with what :func:`backward_from` needs.
+    With ``cfg["norm_eps"]`` set the rows are RMS-normalised (weight ``norm_w`` or none) on the way
+    into the router; the normalised rows then stand for ``x`` in every later stage and in ``saved``."""
     e, k, tile_m = cfg["num_experts"], cfg["top_k"], cfg["tile_m"]
     score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
-    idx, w, logits = _abi.router_topk(x, router, cfg["router_bias"], k, score_fn, renorm, want_logits=True)
+    if cfg.get("norm_eps") is not None:
+        x, idx, w, logits = _abi.router_topk_norm(x, norm_w, cfg["norm_eps"], router, cfg["router_bias"], k,
+                                                  score_fn, renorm, want_logits=True)
+    else:
+        idx, w, logits = _abi.router_topk(x, router, cfg["router_bias"], k, score_fn, renorm, want_logits=True)
     disp = _abi.dispatch(idx, w, x, e, tile_m, scale_input, gather=True)
     # where the expert kernel can, it leaves the gate and the up product behind for the backward
     # pass (what autograd would save); otherwise backward_from computes them again
@@ -62,13 +72,14 @@ def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg):
         else:
             base = _abi.dense_swiglu(x, sg, su, sd)
     out = _abi.combine(ye, disp.inv_perm, idx, w, base, not scale_input, out=base, residual=residual)
-    return out, (idx, w, logits, disp.counts, disp.offsets, disp.inv_perm, disp.xe, ye, g, u, g_s, u_s)
+    xn = x if cfg.get("norm_eps") is not None else None
+    return out, (idx, w, logits, disp.counts, disp.offsets, disp.inv_perm, disp.xe, ye, g, u, g_s, u_s, xn)
 
 
 def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
     """Gradients ``(dx, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd)`` (None where ``need`` -- in
     that order -- says so) from the output gradient and the intermediates of :func:`forward_saving`."""
-    idx, w, logits, counts, offsets, inv_perm, xe, ye, g, u, g_s, u_s = saved
+    idx, w, logits, counts, offsets, inv_perm, xe, ye, g, u, g_s, u_s = saved[:12]
     e, tile_m = cfg["num_experts"], cfg["tile_m"]
     score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
     dout = dout.contiguous()
@@ -151,23 +162,33 @@ def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
 
 
 class MoEFunction(torch.autograd.Function):
-    """``forward(x, residual, router, wg, wu, wd, sg, su, sd, cfg)``; ``cfg`` carries the integers."""
+    """``forward(x, residual, router, wg, wu, wd, sg, su, sd, norm_w, cfg)``; ``cfg`` carries the
+    integers (and ``norm_eps`` when the rows are normalised first; ``norm_w`` may then still be None)."""
 
     @staticmethod
-    def forward(ctx, x, residual, router, wg, wu, wd, sg, su, sd, cfg):  # noqa: D102
-        out, saved = forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg)
+    def forward(ctx, x, residual, router, wg, wu, wd, sg, su, sd, norm_w, cfg):  # noqa: D102
+        out, saved = forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg, norm_w)
         ctx.cfg = cfg
         ctx.has_residual = residual is not None
-        ctx.save_for_backward(x, router, wg, wu, wd, sg, su, sd, *saved)
+        ctx.save_for_backward(x, router, wg, wu, wd, sg, su, sd, norm_w, *saved)
         return out
 
     @staticmethod
     @torch.no_grad()
     def backward(ctx, dout):  # noqa: D102
-        x, router, wg, wu, wd, sg, su, sd, *saved = ctx.saved_tensors
+        x, router, wg, wu, wd, sg, su, sd, norm_w, *saved = ctx.saved_tensors
         n = ctx.needs_input_grad
-        need = (n[0], n[2], n[3], n[4], n[5], n[6], n[7], n[8])
+        normed = ctx.cfg.get("norm_eps") is not None
+        # through the normalisation the rows' gradient is needed for the weight's as well
+        need = (n[0] or (normed and n[9]), n[2], n[3], n[4], n[5], n[6], n[7], n[8])
+        xn = saved[12]
         dx, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd = backward_from(
-            x, router, wg, wu, wd, sg, su, sd, tuple(saved), ctx.cfg, dout, need)
+            xn if normed else x, router, wg, wu, wd, sg, su, sd, tuple(saved), ctx.cfg, dout, need)
+        d_norm_w = None
+        if normed and dx is not None:
+            dx, d_norm_w = _abi.rms_norm_backward(x, norm_w, ctx.cfg["norm_eps"], dx,
+                                                  want_weight_grad=bool(n[9]))
+            if not n[0]:
+                dx = None
         d_res = dout if ctx.has_residual and n[1] else None
-        return dx, d_res, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd, None
+        return dx, d_res, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd, d_norm_w, None

@@ -420,6 +420,130 @@ __global__ __launch_bounds__(256) void pair_dot_kernel(const T* __restrict__ a,
   if (lane == 0) out[p] = s;
 }
 
+// ------------------------------------------------------------------- RMS normalisation backward
+// y = x r w with r = rsqrt(mean(x^2) + eps) (nn/normalization.py:234-236).  With gy = dy w:
+//   dx = r gy - x r^3 <gy, x> / D        dw[j] = sum_t dy[t, j] x[t, j] r_t
+// One wave per row, two passes over it (the second finds the row in cache); everything in f32,
+// one rounding per stored element.  The row's r goes to rstd (may be null) for the weight gradient.
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_backward_rows_kernel(
+    const T* __restrict__ x, const T* __restrict__ w, float eps, const T* __restrict__ dy, int rows,
+    int D, T* __restrict__ dx, float* __restrict__ rstd) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  constexpr int VEC = 16 / sizeof(T);
+  const bool vec = D % VEC == 0;  // the host checks the alignment of the bases
+  const float inv_d = 1.0f / (float)D;
+  for (int t = blockIdx.x * 4 + wave; t < rows; t += gridDim.x * 4) {
+    const T* xr = x + (size_t)t * D;
+    const T* gr = dy + (size_t)t * D;
+    T* outr = dx + (size_t)t * D;
+    float ss = 0.f, sg = 0.f;
+    if (vec) {
+      for (int d = lane * VEC; d < D; d += 64 * VEC) {
+        const u32x4 xv = *reinterpret_cast<const u32x4*>(xr + d);
+        const u32x4 gv = *reinterpret_cast<const u32x4*>(gr + d);
+        u32x4 wv = {0u, 0u, 0u, 0u};
+        if (w != nullptr) wv = *reinterpret_cast<const u32x4*>(w + d);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if constexpr (sizeof(T) == 2) {
+            const float x0 = __uint_as_float(xv[j] << 16), x1 = __uint_as_float(xv[j] & 0xffff0000u);
+            float g0 = __uint_as_float(gv[j] << 16), g1 = __uint_as_float(gv[j] & 0xffff0000u);
+            if (w != nullptr) {
+              g0 *= __uint_as_float(wv[j] << 16);
+              g1 *= __uint_as_float(wv[j] & 0xffff0000u);
+            }
+            ss += x0 * x0;
+            ss += x1 * x1;
+            sg += g0 * x0;
+            sg += g1 * x1;
+          } else {
+            const float x0 = __uint_as_float(xv[j]);
+            float g0 = __uint_as_float(gv[j]);
+            if (w != nullptr) g0 *= __uint_as_float(wv[j]);
+            ss += x0 * x0;
+            sg += g0 * x0;
+          }
+        }
+      }
+    } else {
+      for (int d = lane; d < D; d += 64) {
+        const float x0 = Elem<T>::load(xr + d);
+        float g0 = Elem<T>::load(gr + d);
+        if (w != nullptr) g0 *= Elem<T>::load(w + d);
+        ss += x0 * x0;
+        sg += g0 * x0;
+      }
+    }
+    const float r = 1.0f / sqrtf(wave_sum_f32(ss) * inv_d + eps);
+    const float c = r * r * r * wave_sum_f32(sg) * inv_d;
+    if (rstd != nullptr && lane == 0) rstd[t] = r;
+    if (vec) {
+      for (int d = lane * VEC; d < D; d += 64 * VEC) {
+        const u32x4 xv = *reinterpret_cast<const u32x4*>(xr + d);
+        const u32x4 gv = *reinterpret_cast<const u32x4*>(gr + d);
+        u32x4 wv = {0u, 0u, 0u, 0u};
+        if (w != nullptr) wv = *reinterpret_cast<const u32x4*>(w + d);
+        u32x4 ov;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if constexpr (sizeof(T) == 2) {
+            const float x0 = __uint_as_float(xv[j] << 16), x1 = __uint_as_float(xv[j] & 0xffff0000u);
+            float g0 = __uint_as_float(gv[j] << 16), g1 = __uint_as_float(gv[j] & 0xffff0000u);
+            if (w != nullptr) {
+              g0 *= __uint_as_float(wv[j] << 16);
+              g1 *= __uint_as_float(wv[j] & 0xffff0000u);
+            }
+            ov[j] = pack_bf16x2(r * g0 - x0 * c, r * g1 - x1 * c);
+          } else {
+            const float x0 = __uint_as_float(xv[j]);
+            float g0 = __uint_as_float(gv[j]);
+            if (w != nullptr) g0 *= __uint_as_float(wv[j]);
+            ov[j] = __float_as_uint(r * g0 - x0 * c);
+          }
+        }
+        *reinterpret_cast<u32x4*>(outr + d) = ov;
+      }
+    } else {
+      for (int d = lane; d < D; d += 64) {
+        const float x0 = Elem<T>::load(xr + d);
+        float g0 = Elem<T>::load(gr + d);
+        if (w != nullptr) g0 *= Elem<T>::load(w + d);
+        Elem<T>::store(outr + d, r * g0 - x0 * c);
+      }
+    }
+  }
+}
+
+// Weight gradient, first half: the rows are cut into gridDim.y slabs; a thread owns a column and
+// adds up dy x r over the rows of its slab in ascending order.  partial [slabs][D] f32.
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_backward_weight_kernel(
+    const T* __restrict__ x, const T* __restrict__ dy, const float* __restrict__ rstd, int rows,
+    int D, float* __restrict__ partial) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= D) return;
+  const int per = (rows + gridDim.y - 1) / gridDim.y;
+  const int t0 = blockIdx.y * per;
+  const int t1 = t0 + per < rows ? t0 + per : rows;
+  float acc = 0.f;
+  for (int t = t0; t < t1; ++t)
+    acc += Elem<T>::load(dy + (size_t)t * D + j) * Elem<T>::load(x + (size_t)t * D + j) * rstd[t];
+  partial[(size_t)blockIdx.y * D + j] = acc;
+}
+
+// Second half: the slabs added in ascending order, one rounding.
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_backward_weight_sum_kernel(
+    const float* __restrict__ partial, int slabs, int D, T* __restrict__ dw) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= D) return;
+  float acc = 0.f;
+  for (int s = 0; s < slabs; ++s) acc += partial[(size_t)s * D + j];
+  Elem<T>::store(dw + j, acc);
+}
+
 // --------------------------------------------------------------------------------- router backward
 // One wave per token: dw [K] -> dlogits [E] (zero where the score function does not reach).
 //   sigmoid:              w_k = s_k,            s = sigmoid(l_k)    dl_k = dw_k s_k (1 - s_k)
@@ -651,4 +775,75 @@ extern "C" int fs2moe_router_backward(const float* logits, const int32_t* topk_i
                        topk_idx, topk_w, d_w, T, E, K, score_fn, renormalize,
                        static_cast<float*>(dlogits));
   return check_launch("router_backward");
+}
+
+// slabs of rows for the weight gradient of the normalisation: at least 32 rows each, at most 64
+static int norm_weight_slabs(int64_t rows) {
+  const int64_t s = rows / 32;
+  return s < 1 ? 1 : (s > 64 ? 64 : (int)s);
+}
+
+extern "C" int64_t fs2moe_rms_norm_backward_workspace_bytes(int32_t T, int32_t D) {
+  if (T < 0 || D < 1) return -1;
+  // rstd [T] (padded to 16 bytes), then the slabs' partial sums
+  return ((int64_t)T * 4 + 15) / 16 * 16 + (int64_t)norm_weight_slabs(T) * D * 4;
+}
+
+extern "C" int fs2moe_rms_norm_backward(const void* x, const void* weight, float eps,
+                                        const void* dy, int32_t T, int32_t D, int32_t dtype,
+                                        void* dx, void* dweight, void* workspace,
+                                        int64_t workspace_bytes, void* stream) {
+  FS2_REQUIRE(x && dy && dx, "rms_norm_backward: null pointer");
+  FS2_REQUIRE(dtype == FS2MOE_F32 || dtype == FS2MOE_BF16, "rms_norm_backward: dtype %d", dtype);
+  FS2_REQUIRE(T >= 0 && D > 0, "rms_norm_backward: T=%d, D=%d", T, D);
+  FS2_REQUIRE(dweight == nullptr || weight != nullptr,
+              "rms_norm_backward: a weight gradient without a weight");
+  FS2_REQUIRE(dx != dy && dx != x, "rms_norm_backward: dx must not alias x or dy");
+  FS2_REQUIRE(aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(weight) &&
+                  aligned16(workspace),
+              "rms_norm_backward: buffers must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* rstd = nullptr;
+  float* partial = nullptr;
+  if (dweight != nullptr) {
+    FS2_REQUIRE(workspace != nullptr &&
+                    workspace_bytes >= fs2moe_rms_norm_backward_workspace_bytes(T, D),
+                "rms_norm_backward: the weight gradient needs a workspace of %lld bytes",
+                (long long)fs2moe_rms_norm_backward_workspace_bytes(T, D));
+    rstd = static_cast<float*>(workspace);
+    partial = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) +
+                                       ((int64_t)T * 4 + 15) / 16 * 16);
+  }
+  if (T > 0) {
+    int blocks = (T + 3) / 4;
+    if (blocks > 4096) blocks = 4096;
+    if (dtype == FS2MOE_BF16)
+      hipLaunchKernelGGL(rms_norm_backward_rows_kernel<uint16_t>, dim3((unsigned)blocks), dim3(256),
+                         0, st, static_cast<const uint16_t*>(x),
+                         static_cast<const uint16_t*>(weight), eps,
+                         static_cast<const uint16_t*>(dy), T, D, static_cast<uint16_t*>(dx), rstd);
+    else
+      hipLaunchKernelGGL(rms_norm_backward_rows_kernel<float>, dim3((unsigned)blocks), dim3(256), 0,
+                         st, static_cast<const float*>(x), static_cast<const float*>(weight), eps,
+                         static_cast<const float*>(dy), T, D, static_cast<float*>(dx), rstd);
+    if (int rc = check_launch("rms_norm_backward")) return rc;
+  }
+  if (dweight == nullptr) return FS2MOE_OK;
+  // (with no rows the one slab sums nothing and the gradient is zero)
+  const int slabs = norm_weight_slabs(T);
+  const dim3 grid((unsigned)((D + 255) / 256), (unsigned)slabs);
+  if (dtype == FS2MOE_BF16) {
+    hipLaunchKernelGGL(rms_norm_backward_weight_kernel<uint16_t>, grid, dim3(256), 0, st,
+                       static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(dy), rstd, T, D,
+                       partial);
+    hipLaunchKernelGGL(rms_norm_backward_weight_sum_kernel<uint16_t>, dim3(grid.x), dim3(256), 0, st,
+                       partial, slabs, D, static_cast<uint16_t*>(dweight));
+  } else {
+    hipLaunchKernelGGL(rms_norm_backward_weight_kernel<float>, grid, dim3(256), 0, st,
+                       static_cast<const float*>(x), static_cast<const float*>(dy), rstd, T, D,
+                       partial);
+    hipLaunchKernelGGL(rms_norm_backward_weight_sum_kernel<float>, dim3(grid.x), dim3(256), 0, st,
+                       partial, slabs, D, static_cast<float*>(dweight));
+  }
+  return check_launch("rms_norm_backward (weight)");
 }

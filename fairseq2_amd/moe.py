@@ -428,7 +428,8 @@ class MoE(FeedForwardNetwork):
         if residual is not None:
             residual = self._autocast(residual)
         wants_grad = torch.is_grad_enabled() and any(
-            t is not None and t.requires_grad for t in (seqs, residual, *self.parameters())
+            isinstance(t, Tensor) and t.requires_grad
+            for t in (seqs, residual, getattr(norm, "weight", None), *self.parameters())
         )
         if wants_grad and not torch.compiler.is_compiling():
             return self._differentiable(seqs, residual, norm)
@@ -460,13 +461,11 @@ class MoE(FeedForwardNetwork):
     def _differentiable(self, seqs: Tensor, residual: Tensor | None, norm) -> Tensor:
         """The training path: the layer as one ``torch.autograd.Function`` whose backward pass runs
         on the library's kernels (:mod:`fairseq2_amd.autograd`), for ``seqs``, ``residual`` and
-        every parameter.  Covers the reference configuration and the routing extensions; the fused
-        normalisation, e4m3 weights and other expert modules are forward-only."""
+        every parameter (the weight of ``norm`` included).  Covers the reference configuration and
+        the extensions; e4m3 weights and other expert modules are forward-only."""
         ex, se = self.experts, self.shared_expert
         why = None
-        if norm is not None:
-            why = "the normalisation fused into the router has no backward pass (normalise outside the layer)"
-        elif type(ex) is not GroupedExpertNetwork or (se is not None and type(se) is not GLUFeedForwardNetwork):
+        if type(ex) is not GroupedExpertNetwork or (se is not None and type(se) is not GLUFeedForwardNetwork):
             why = "only GroupedExpertNetwork experts and a GLUFeedForwardNetwork shared expert are differentiated"
         elif not ex.has_fused_gate and any(p.requires_grad for p in ex.activation.parameters()):
             why = "a gate activation with parameters of its own is not differentiated"
@@ -477,6 +476,7 @@ class MoE(FeedForwardNetwork):
                 f"fairseq2_amd.MoE: {why}; call it under torch.no_grad() / torch.inference_mode(), "
                 "or freeze the inputs and the module with requires_grad_(False)")
         x = self._checked_rows(seqs, allow_grad=True)
+        norm_args = self._norm_args(norm, x, allow_grad=True)
         res = None
         if residual is not None:
             if residual.shape != seqs.shape or residual.dtype != seqs.dtype:
@@ -500,9 +500,10 @@ class MoE(FeedForwardNetwork):
             score_fn=_SCORE_FNS[self.score_fn], renormalize=self.renormalize,
             scale_input=self.scale_on == "input", router_bias=self.router_bias,
             activation=None if ex.has_fused_gate else ex.activation,
+            norm_eps=None if norm_args is None else norm_args[1],
         )
         out = MoEFunction.apply(x, res, self.router, ex.gate_proj, ex.inner_proj, ex.output_proj,
-                                *shared, cfg)
+                                *shared, None if norm_args is None else norm_args[0], cfg)
         return out.view(seqs.shape)
 
     def _autocast(self, t: Tensor) -> Tensor:
@@ -513,8 +514,9 @@ class MoE(FeedForwardNetwork):
         return t
 
     @staticmethod
-    def _norm_args(norm, x: Tensor) -> tuple[Tensor | None, float] | None:
-        """(weight, eps) of an RMS normalisation module, checked against the rows ``x``."""
+    def _norm_args(norm, x: Tensor, allow_grad: bool = False) -> tuple[Tensor | None, float] | None:
+        """(weight, eps) of an RMS normalisation module, checked against the rows ``x``; the weight
+        detached unless ``allow_grad`` (the training path differentiates it)."""
         if norm is None:
             return None
         if getattr(norm, "bias", None) is not None:
@@ -525,10 +527,11 @@ class MoE(FeedForwardNetwork):
         weight = getattr(norm, "weight", None)
         if weight is not None:
             _require_device(weight)
-            _require_forward_only(weight)
+            if not allow_grad:
+                _require_forward_only(weight)
             if weight.dtype != x.dtype or weight.shape != (x.shape[-1],):
                 raise ValueError("the norm weight must be (dim,) in the dtype of seqs")
-            weight = weight.detach().contiguous()
+            weight = (weight if allow_grad else weight.detach()).contiguous()
         return weight, float(norm.eps)
 
     def _single_call(self, x: Tensor, residual: Tensor | None = None, norm=None) -> Tensor:

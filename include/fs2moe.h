@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FS2MOE_ABI_VERSION 10
+#define FS2MOE_ABI_VERSION 11
 
 /* element types */
 #define FS2MOE_F32 0
@@ -360,6 +360,23 @@ int fs2moe_pair_dot(const void* a, const void* a2, const int32_t* a_rows, const 
 int fs2moe_router_backward(const float* logits, const int32_t* topk_idx, const float* topk_w,
                            const float* d_w, int32_t T, int32_t E, int32_t K, int32_t score_fn,
                            int32_t renormalize, int32_t dtype, void* dlogits, void* stream);
+
+/*
+ * Backward of the RMS normalisation that fs2moe_router_topk_norm / fs2moe_forward_norm put in front
+ * of the layer: y = x * rsqrt(mean(x^2) + eps) * weight.  What autograd derives for
+ * torch.nn.functional.rms_norm (nn/normalization.py:234-236), the ffn_layer_norm call of
+ * models/transformer_lm/decoder_layer.py:187-191.
+ *   dx[t] = r_t * (dy[t] * weight) - x[t] * r_t^3 * <dy[t] * weight, x[t]> / D
+ *   dweight[j] = sum over t (ascending, in up to 64 slabs) of dy[t, j] * x[t, j] * r_t
+ * all in f32 with one rounding per stored element.
+ *   x, dy [T, D] dtype   weight [D] dtype or NULL   dx [T, D] dtype (out; must not alias x or dy)
+ *   dweight [D] dtype (out) or NULL; when given, workspace must hold
+ *   fs2moe_rms_norm_backward_workspace_bytes(T, D) bytes (16-byte aligned); otherwise it is unused.
+ */
+int64_t fs2moe_rms_norm_backward_workspace_bytes(int32_t T, int32_t D);
+int fs2moe_rms_norm_backward(const void* x, const void* weight, float eps, const void* dy,
+                             int32_t T, int32_t D, int32_t dtype, void* dx, void* dweight,
+                             void* workspace, int64_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

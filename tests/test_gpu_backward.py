@@ -18,7 +18,7 @@ import torch
 from fairseq2_amd import _abi
 import workloads as W
 from oracle import moe_oracle as O
-from tests._util import TORCH_DTYPE, build_module
+from tests._util import TORCH_DTYPE, assert_output_close, build_module
 
 pytestmark = pytest.mark.gpu
 
@@ -432,6 +432,121 @@ def test_gradients_with_a_number_of_experts_that_is_not_a_multiple_of_8(gpu_devi
         assert_grad_close(p.grad, ref[name], dtype, f"d {name}")
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("t,d,with_weight", [(1, 64, True), (37, 200, True), (300, 2048, True), (129, 72, False),
+                                             (5, 4104, True), (70, 100, True), (2100, 256, True)])
+def test_rms_norm_backward_matches_autograd_of_the_oracle(gpu_device, dtype, t, d, with_weight):
+    """``fs2moe_rms_norm_backward`` against float64 autograd through the oracle's restatement of
+    ``torch.nn.functional.rms_norm`` (``nn/normalization.py:234-236``)."""
+    dt = TORCH_DTYPE[dtype]
+    g = torch.Generator().manual_seed(t * 1000 + d)
+    x = (torch.randn(t, d, generator=g) * 1.7 + 0.3).to(dt)
+    w = (1.0 + 0.2 * torch.randn(d, generator=g)).to(dt) if with_weight else None
+    dy = torch.randn(t, d, generator=g).to(dt)
+    eps = 1e-5
+    x64 = x.double().requires_grad_(True)
+    w64 = None if w is None else w.double().requires_grad_(True)
+    O.rms_norm(x64, w64, eps).backward(dy.double())
+    dx, dw = _abi.rms_norm_backward(x.to(gpu_device), None if w is None else w.to(gpu_device), eps,
+                                    dy.to(gpu_device))
+    assert_grad_close(dx, x64.grad, dtype, "d x")
+    if w is None:
+        assert dw is None
+    else:
+        assert_grad_close(dw, w64.grad, dtype, "d weight")
+        # without the weight's gradient the rows' is the same, bit for bit, and needs no scratch
+        dx2, none = _abi.rms_norm_backward(x.to(gpu_device), w.to(gpu_device), eps, dy.to(gpu_device),
+                                           want_weight_grad=False)
+        assert none is None and torch.equal(dx2, dx)
+
+
+class _RMSNorm(torch.nn.Module):
+    """What the layer reads of ``fairseq2.nn.RMSNorm`` (``nn/normalization.py:166-254``)."""
+
+    def __init__(self, dim, dtype, device, weight=True):
+        super().__init__()
+        g = torch.Generator().manual_seed(dim)
+        self.weight = torch.nn.Parameter((1.0 + 0.2 * torch.randn(dim, generator=g)).to(dtype).to(device)) if weight else None
+        self.bias, self.eps, self.normalized_shape = None, 1e-5, (dim,)
+
+
+@pytest.mark.parametrize("mode,shared,with_weight", [("reference", True, True), ("softmax_renorm_output", False, True),
+                                                     ("reference", False, False)])
+def test_gradients_through_the_normalisation_in_front_fp32(gpu_device, mode, shared, with_weight):
+    """``layer(seqs, residual=seqs, norm=layer_norm)`` in training (the feed-forward half of a
+    pre-norm decoder layer, ``decoder_layer.py:187-204``) against float64 autograd through the
+    oracle's norm and the dense restatement of the layer.  f32 only: in bf16 the device routes the
+    rounded normalised rows, whose near-ties the float64 path resolves differently (the bf16 case
+    is the composition test below)."""
+    spec = W.small_spec(tokens=300, model_dim=128, num_experts=16, top_k=2, inner_dim=96, dtype="fp32",
+                        shared=shared, zipf_s=1.0, mode=MODES[mode], seed=41)
+    wl = W.make_workload_from_spec(spec)
+    m = build_module(wl, gpu_device).train().requires_grad_(True)
+    norm = _RMSNorm(spec.model_dim, torch.float32, gpu_device, with_weight)
+    g = torch.Generator().manual_seed(8)
+    grad_out = torch.randn(wl.x.shape, generator=g)
+    # reference: the norm in float64 in front of the dense restatement, the raw rows as residual
+    s = wl.spec
+    c = lambda t: None if t is None else t.double().clone().requires_grad_(True)  # noqa: E731
+    x, router, gate, up, down = c(wl.x), c(wl.router), c(wl.gate), c(wl.up), c(wl.down)
+    sh = (c(wl.shared_gate), c(wl.shared_up), c(wl.shared_down)) if s.shared else None
+    nw = None if norm.weight is None else c(norm.weight.detach().cpu())
+    out = x + O.ref_dense_forward(
+        O.rms_norm(x, nw, norm.eps), router, gate, up, down, s.top_k, shared=sh,
+        router_bias=None if wl.router_bias is None else wl.router_bias.double(),
+        score_fn=s.mode.score_fn, renormalize=s.mode.renormalize, scale_on=s.mode.scale_on)
+    out.backward(grad_out.double())
+    xd = wl.x.to(gpu_device).requires_grad_(True)
+    got = m(xd, residual=xd, norm=norm)
+    assert_output_close(got, out.detach(), "fp32", "pre-norm layer, training path")
+    got.backward(grad_out.to(gpu_device))
+    assert_grad_close(xd.grad, x.grad, "fp32", "d x")
+    if nw is not None:
+        assert_grad_close(norm.weight.grad, nw.grad, "fp32", "d norm weight")
+    ref = {"router": router.grad, "experts.gate_proj": gate.grad, "experts.inner_proj": up.grad,
+           "experts.output_proj": down.grad}
+    if sh is not None:
+        ref.update({"shared_expert.gate_proj.weight": sh[0].grad, "shared_expert.inner_proj.weight": sh[1].grad,
+                    "shared_expert.output_proj.weight": sh[2].grad})
+    for name, p in m.named_parameters():
+        assert_grad_close(p.grad, ref[name], "fp32", f"d {name}")
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_gradients_through_the_normalisation_compose(gpu_device, dtype):
+    """The same call in bf16, checked piece by piece on the device's own normalised rows: the
+    layer's gradients are those of the layer without ``norm`` on ``xn`` (bit for bit: same kernels,
+    same inputs), and the rows' gradient is ``fs2moe_rms_norm_backward`` of that layer's input
+    gradient plus the residual's.  (Each piece is checked against the oracle by its own test.)"""
+    dt = TORCH_DTYPE[dtype]
+    spec = W.small_spec(tokens=700, model_dim=256, num_experts=16, top_k=4, inner_dim=128, dtype=dtype,
+                        shared=True, zipf_s=1.0, seed=43)
+    wl = W.make_workload_from_spec(spec)
+    m = build_module(wl, gpu_device).train().requires_grad_(True)
+    norm = _RMSNorm(spec.model_dim, dt, gpu_device)
+    g = torch.Generator().manual_seed(9)
+    grad_out = torch.randn(wl.x.shape, generator=g).to(dt).to(gpu_device)
+    xd = wl.x.to(dt).to(gpu_device).requires_grad_(True)
+    out = m(xd, residual=xd, norm=norm)
+    with torch.no_grad():
+        assert torch.equal(out, m(xd, residual=xd, norm=norm))  # the inference path's values
+    out.backward(grad_out)
+    got = {n: p.grad.clone() for n, p in m.named_parameters()}
+    got_x, got_nw = xd.grad.clone(), norm.weight.grad.clone()
+    m.zero_grad()
+    rows = xd.detach().reshape(-1, spec.model_dim)
+    xn = _abi.router_topk_norm(rows, norm.weight.detach(), norm.eps, m.router.detach(), m.router_bias,
+                               m.top_k)[0].requires_grad_(True)
+    m(xn).backward(grad_out.reshape(xn.shape))
+    for n, p in m.named_parameters():
+        assert torch.equal(p.grad, got[n]), n
+    dx, dnw = _abi.rms_norm_backward(rows, norm.weight.detach(), norm.eps, xn.grad)
+    assert torch.equal(dnw, got_nw)
+    want_x = (dx.float() + grad_out.reshape(xn.shape).float()).to(dt).view(got_x.shape)
+    # autograd adds the two gradients of xd in the tensors' dtype: one more rounding than want_x has
+    torch.testing.assert_close(got_x.float(), want_x.float(), rtol=2 ** -7 if dtype == "bf16" else 1e-6, atol=1e-6)
+
+
 def test_frozen_parameters_get_no_gradient_and_unsupported_cases_say_so(gpu_device):
     wl = W.make_workload_from_spec(W.small_spec(dtype="bf16", tokens=64, num_experts=8, inner_dim=128, seed=3))
     m = build_module(wl, gpu_device)  # frozen
@@ -440,11 +555,6 @@ def test_frozen_parameters_get_no_gradient_and_unsupported_cases_say_so(gpu_devi
     out.sum().backward()
     assert x.grad is not None and all(p.grad is None for p in m.parameters())
 
-    class _Norm:
-        weight, bias, eps, normalized_shape = None, None, 1e-5, (wl.spec.model_dim,)
-
-    with pytest.raises(RuntimeError, match="no backward pass"):
-        m(x, norm=_Norm)
     m.experts.activation = torch.nn.PReLU().to(gpu_device)
     with pytest.raises(RuntimeError, match="parameters of its own"):
         m(x)
