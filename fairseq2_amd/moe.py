@@ -436,7 +436,7 @@ class MoE(FeedForwardNetwork):
         # (while a compiler traces the call, training goes through the registered operator below,
         # which carries its own autograd formula)
         x = self._checked_rows(seqs, allow_grad=wants_grad)
-        norm_args = self._norm_args(norm, x)
+        norm_args = self._norm_args(norm, x, allow_grad=wants_grad)
         res = None
         if residual is not None:
             if residual.shape != seqs.shape or residual.dtype != seqs.dtype:

@@ -8,8 +8,8 @@ one, the whole-layer entry point of the library, for the GPU.  Outside a trace t
 library directly (an operator dispatch costs more host time than a decode-sized layer takes).
 
 Training under ``torch.compile``: the operator has an autograd formula, a second registered operator
-``torch.ops.fairseq2_amd.moe_backward`` that recomputes the forward pass's intermediates (routing,
-gathered rows, expert outputs) and runs the backward kernels of :mod:`fairseq2_amd.autograd`; a
+``torch.ops.fairseq2_amd.moe_backward`` that recomputes the forward pass's intermediates (normalised
+rows, routing, gathered rows, expert outputs) and runs the backward kernels of :mod:`fairseq2_amd.autograd`; a
 compiled layer therefore stays one graph in training as well, for the recomputation's price.  Eager
 training does not pay it (the module keeps the intermediates of its own forward pass).
 """
@@ -83,26 +83,36 @@ def moe_backward(
     score_fn: int,
     renormalize: bool,
     scale_input: bool,
+    norm_weight: Optional[Tensor],
+    normed: bool,
+    norm_eps: float,
 ) -> list[Tensor]:
-    """Gradients of ``moe_forward`` for ``x``, ``router``, the three expert weights and (when given)
-    the three shared-expert weights, in that order (5 or 8 tensors)."""
+    """Gradients of ``moe_forward`` for ``x``, ``router``, the three expert weights, (when given)
+    the three shared-expert weights and (when given) the norm's weight, in that order."""
     from fairseq2_amd.autograd import backward_from, forward_saving
 
     cfg = dict(num_experts=num_experts, top_k=top_k, tile_m=tile_m, score_fn=score_fn,
-               renormalize=renormalize, scale_input=scale_input, router_bias=router_bias)
+               renormalize=renormalize, scale_input=scale_input, router_bias=router_bias,
+               norm_eps=norm_eps if normed else None)
     _, saved = forward_saving(x, None, router, w_gate, w_up, w_down, shared_gate, shared_up,
-                              shared_down, cfg)
-    grads = backward_from(x, router, w_gate, w_up, w_down, shared_gate, shared_up, shared_down,
-                          saved, cfg, grad_out, (True,) * 8)
+                              shared_down, cfg, norm_weight)
+    grads = list(backward_from(saved[12] if normed else x, router, w_gate, w_up, w_down, shared_gate,
+                               shared_up, shared_down, saved, cfg, grad_out, (True,) * 8))
+    if normed:
+        grads[0], d_norm_w = _abi.rms_norm_backward(x, norm_weight, norm_eps, grads[0])
+        grads.append(d_norm_w)
     return [g for g in grads if g is not None]
 
 
 @moe_backward.register_fake
 def _moe_backward_fake(grad_out, x, router, router_bias, w_gate, w_up, w_down, shared_gate,
-                       shared_up, shared_down, *ints):
+                       shared_up, shared_down, num_experts, top_k, tile_m, score_fn, renormalize,
+                       scale_input, norm_weight, normed, norm_eps):
     out = [torch.empty_like(t) for t in (x, router, w_gate, w_up, w_down)]
     if shared_gate is not None:
         out += [torch.empty_like(t) for t in (shared_gate, shared_up, shared_down)]
+    if normed and norm_weight is not None:
+        out.append(torch.empty_like(norm_weight))
     return out
 
 
@@ -110,27 +120,32 @@ def _setup_context(ctx, inputs, output):
     (x, router, router_bias, w_gate, w_up, w_down, s_gate, s_up, s_down, shared_gate, shared_up,
      shared_down, residual, norm_weight, num_experts, top_k, tile_m, score_fn, renormalize,
      scale_input, normed, norm_eps) = inputs
-    if s_gate is not None or normed:
-        ctx.unsupported = "e4m3 weights and the fused normalisation are forward-only"
+    if s_gate is not None:
+        ctx.unsupported = "e4m3 weights are forward-only"
         return
     ctx.unsupported = None
     ctx.ints = (num_experts, top_k, tile_m, score_fn, renormalize, scale_input)
+    ctx.norm = (normed, norm_eps)
     ctx.has_residual = residual is not None
     ctx.has_shared = shared_gate is not None
-    ctx.save_for_backward(x, router, router_bias, w_gate, w_up, w_down, shared_gate, shared_up, shared_down)
+    ctx.has_norm_weight = normed and norm_weight is not None
+    ctx.save_for_backward(x, router, router_bias, w_gate, w_up, w_down, shared_gate, shared_up,
+                          shared_down, norm_weight if normed else None)
 
 
 def _backward(ctx, grad_out):
     if ctx.unsupported is not None:
         raise RuntimeError(f"fairseq2_amd::moe_forward: {ctx.unsupported}")
-    x, router, router_bias, w_gate, w_up, w_down, sg, su, sd = ctx.saved_tensors
+    x, router, router_bias, w_gate, w_up, w_down, sg, su, sd, norm_w = ctx.saved_tensors
     grads = torch.ops.fairseq2_amd.moe_backward(
-        grad_out.contiguous(), x, router, router_bias, w_gate, w_up, w_down, sg, su, sd, *ctx.ints)
+        grad_out.contiguous(), x, router, router_bias, w_gate, w_up, w_down, sg, su, sd, *ctx.ints,
+        norm_w, *ctx.norm)
     dx, d_router, d_wg, d_wu, d_wd = grads[:5]
     d_sg, d_su, d_sd = grads[5:8] if ctx.has_shared else (None, None, None)
+    d_norm_w = grads[-1] if ctx.has_norm_weight else None
     d_res = grad_out if ctx.has_residual else None
     # one entry per argument of moe_forward
-    return (dx, d_router, None, d_wg, d_wu, d_wd, None, None, None, d_sg, d_su, d_sd, d_res, None,
+    return (dx, d_router, None, d_wg, d_wu, d_wd, None, None, None, d_sg, d_su, d_sd, d_res, d_norm_w,
             None, None, None, None, None, None, None, None)
 
 

@@ -564,8 +564,8 @@ def test_frozen_parameters_get_no_gradient_and_unsupported_cases_say_so(gpu_devi
         m(x)
 
 
-@pytest.mark.parametrize("shared,with_residual", [(False, False), (True, True)])
-def test_training_step_under_torch_compile(gpu_device, shared, with_residual):
+@pytest.mark.parametrize("shared,with_residual,with_norm", [(False, False, False), (True, True, False), (True, True, True)])
+def test_training_step_under_torch_compile(gpu_device, shared, with_residual, with_norm):
     """A compiled layer in training mode (transformer_lm/compiler.py:14-17 wraps layers that the
     trainer then differentiates): the registered operator carries an autograd formula, so the trace is
     one graph, and its gradients are those of the eager training path (same kernels: bit-equal)."""
@@ -578,14 +578,18 @@ def test_training_step_under_torch_compile(gpu_device, shared, with_residual):
 
     def grads(compiled):
         m = build_module(wl, gpu_device).train().requires_grad_(True)
+        norm = _RMSNorm(spec.model_dim, torch.bfloat16, gpu_device) if with_norm else None
         x = wl.x.to(torch.bfloat16).to(gpu_device).requires_grad_(True)
-        fn = (lambda t: m(t, residual=t)) if with_residual else (lambda t: m(t))  # noqa: E731
+        fn = (lambda t: m(t, residual=t, norm=norm)) if with_residual else (lambda t: m(t))  # noqa: E731
         if compiled:
             fn = torch.compile(fn, backend="aot_eager", fullgraph=True)
         out = fn(x)
         out.backward(g)
         torch.cuda.synchronize()
-        return out.detach(), x.grad, {n: p.grad for n, p in m.named_parameters()}
+        params = {n: p.grad for n, p in m.named_parameters()}
+        if norm is not None:
+            params["norm.weight"] = norm.weight.grad
+        return out.detach(), x.grad, params
 
     out_e, dx_e, dp_e = grads(False)
     out_c, dx_c, dp_c = grads(True)

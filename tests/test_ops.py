@@ -35,9 +35,14 @@ def test_backward_operator_is_registered_with_a_shape_only_implementation():
     with FakeTensorMode():
         a = _args("cuda")
         x, router, _, w_in, _, w_out = a[:6]
-        grads = op(torch.empty_like(x), x, router, None, w_in, w_in, w_out, None, None, None, 8, 2, 16, 0, False, True)
+        grads = op(torch.empty_like(x), x, router, None, w_in, w_in, w_out, None, None, None, 8, 2, 16, 0, False, True, None, False, 0.0)
         assert [g.shape for g in grads] == [x.shape, router.shape, w_in.shape, w_in.shape, w_out.shape]
         sg = torch.empty(32, 64, device="cuda", dtype=torch.bfloat16)
         sd = torch.empty(64, 32, device="cuda", dtype=torch.bfloat16)
-        grads = op(torch.empty_like(x), x, router, None, w_in, w_in, w_out, sg, sg, sd, 8, 2, 16, 0, False, True)
+        grads = op(torch.empty_like(x), x, router, None, w_in, w_in, w_out, sg, sg, sd, 8, 2, 16, 0, False, True,
+                   None, False, 0.0)
         assert len(grads) == 8 and grads[7].shape == sd.shape
+        nw = torch.empty(64, device="cuda", dtype=torch.bfloat16)
+        grads = op(torch.empty_like(x), x, router, None, w_in, w_in, w_out, sg, sg, sd, 8, 2, 16, 0, False, True,
+                   nw, True, 1e-5)
+        assert len(grads) == 9 and grads[8].shape == nw.shape
