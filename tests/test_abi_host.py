@@ -137,6 +137,62 @@ def test_argument_errors_are_reported_without_touching_the_gpu(lib):
     assert lib.fs2moe_dispatch_workspace_bytes(-1, 8, 128) == -1
 
 
+def test_backward_entry_points_report_argument_errors_without_touching_the_gpu(lib):
+    fake, other = ctypes.c_void_p(0x1000), ctypes.c_void_p(0x2000)
+    err = lib.fs2moe_last_error
+    # plain grouped product: layout, sizes, groups
+    rc = lib.fs2moe_grouped_gemm(fake, None, fake, fake, fake, 7, 4, 64, 64, 128, _abi.BF16, fake, None)
+    assert rc == -1 and b"layout" in err()
+    rc = lib.fs2moe_grouped_gemm(fake, None, fake, fake, fake, _abi.W_IN_OUT, 4, 60, 64, 128, _abi.BF16, fake, None)
+    assert rc == -1 and b"multiples of 8" in err()
+    rc = lib.fs2moe_grouped_gemm(fake, None, fake, None, fake, _abi.W_IN_OUT, 4, 64, 64, 128, _abi.BF16, fake, None)
+    assert rc == -1 and b"counts without offsets" in err()
+    rc = lib.fs2moe_grouped_gemm(fake, None, None, None, fake, _abi.W_IN_OUT, 4, 64, 64, 128, _abi.BF16, fake, None)
+    assert rc == -1 and b"E=4" in err()  # one matrix without groups
+    assert lib.fs2moe_grouped_gemm(fake, None, fake, fake, fake, _abi.W_IN_OUT, 4, 64, 64, 0, _abi.BF16, fake, None) == 0
+    # two-source product: only where the throughput kernel runs
+    assert lib.fs2moe_grouped_gemm_sum_supported(768, 2048, 65536, _abi.BF16) == 1
+    assert lib.fs2moe_grouped_gemm_sum_supported(768, 2048, 65536, _abi.F32) == 0
+    assert lib.fs2moe_grouped_gemm_sum_supported(760, 2048, 65536, _abi.BF16) == 0
+    rc = lib.fs2moe_grouped_gemm_sum(fake, fake, fake, fake, fake, fake, 4, 760, 2048, 1024, _abi.BF16, fake, None)
+    assert rc != 0 and b"grouped_gemm_sum" in err()
+    # kept products: bf16 with the throughput kernel's sizes only
+    assert lib.fs2moe_grouped_swiglu_keeps(2048, 768, 65536, _abi.BF16) == 1
+    assert lib.fs2moe_grouped_swiglu_keeps(2048, 768, 65536, _abi.F32) == 0
+    assert lib.fs2moe_grouped_swiglu_keeps(2048, 760, 65536, _abi.BF16) == 0
+    # weight gradient
+    rc = lib.fs2moe_grouped_wgrad(fake, None, fake, fake, fake, 4, 60, 64, 128, _abi.BF16, fake, None, 0, None)
+    assert rc == -1 and b"multiples of 8" in err()
+    rc = lib.fs2moe_grouped_wgrad(fake, None, fake, fake, fake, 4, 64, 64, 128, 9, fake, None, 0, None)
+    assert rc == -1 and b"dtype 9" in err()
+    assert lib.fs2moe_grouped_wgrad_workspace_bytes(1, 2048, 128, 8192) == 0
+    assert lib.fs2moe_grouped_wgrad_workspace_bytes(0, 2048, 128, 8192) > 0  # the router's gradient: segments
+    assert lib.fs2moe_grouped_wgrad_workspace_bytes(0, 0, 128, 8192) == -1
+    # element-wise and per-token steps
+    rc = lib.fs2moe_swiglu_backward(fake, fake, fake, 10, 60, _abi.BF16, fake, fake, fake, None)
+    assert rc == -1 and b"F=60" in err()
+    rc = lib.fs2moe_pair_dot(fake, None, fake, fake, 4, 17, 64, _abi.BF16, fake, None)
+    assert rc == -1 and b"K=17" in err()
+    rc = lib.fs2moe_router_backward(fake, fake, fake, fake, 4, 1000, 2, 0, 0, _abi.BF16, fake, None)
+    assert rc == -1 and b"E=1000" in err()
+    rc = lib.fs2moe_router_backward(fake, fake, fake, fake, 4, 8, 2, 5, 0, _abi.BF16, fake, None)
+    assert rc == -1 and b"score_fn 5" in err()
+    # the normalisation's backward: no aliasing, the weight's gradient needs the weight and scratch
+    need = lib.fs2moe_rms_norm_backward_workspace_bytes(100, 64)
+    assert need >= 100 * 4 + 3 * 64 * 4 and lib.fs2moe_rms_norm_backward_workspace_bytes(100, 0) == -1
+    rc = lib.fs2moe_rms_norm_backward(fake, None, 1e-5, other, 100, 64, _abi.BF16, other, None, None, 0, None)
+    assert rc == -1 and b"alias" in err()
+    out = ctypes.c_void_p(0x3000)
+    rc = lib.fs2moe_rms_norm_backward(fake, None, 1e-5, other, 100, 64, _abi.BF16, out, fake, fake, need, None)
+    assert rc == -1 and b"without a weight" in err()
+    rc = lib.fs2moe_rms_norm_backward(fake, fake, 1e-5, other, 100, 64, _abi.BF16, out, fake, fake, need - 1, None)
+    assert rc == -1 and b"workspace" in err()
+    rc = lib.fs2moe_rms_norm_backward(fake, fake, 1e-5, other, 100, 64, 9, out, None, None, 0, None)
+    assert rc == -1 and b"dtype 9" in err()
+    # no rows and no weight gradient: nothing to launch
+    assert lib.fs2moe_rms_norm_backward(fake, fake, 1e-5, other, 0, 64, _abi.BF16, out, None, None, 0, None) == 0
+
+
 def test_max_rows_matches_the_header_macro():
     # FS2MOE_MAX_ROWS(T, K, E, tile_m) = T*K + E*(tile_m - 1)
     assert _abi.max_rows(8192, 8, 128, 16) == 8192 * 8 + 128 * 15
