@@ -516,32 +516,70 @@ __global__ __launch_bounds__(256) void rms_norm_backward_rows_kernel(
   }
 }
 
-// Weight gradient, first half: the rows are cut into gridDim.y slabs; a thread owns a column and
-// adds up dy x r over the rows of its slab in ascending order.  partial [slabs][D] f32.
+// Weight gradient, first half: the rows are cut into gridDim.y slabs; a thread owns 16 bytes' worth
+// of columns (one column when D does not divide that way) and adds up dy x r over the rows of its
+// slab in ascending order.  partial [slabs][D] f32.
 template <typename T>
 __global__ __launch_bounds__(256) void rms_norm_backward_weight_kernel(
     const T* __restrict__ x, const T* __restrict__ dy, const float* __restrict__ rstd, int rows,
     int D, float* __restrict__ partial) {
-  const int j = blockIdx.x * 256 + threadIdx.x;
-  if (j >= D) return;
+  constexpr int VEC = 16 / sizeof(T);
+  const bool vec = D % VEC == 0;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= (vec ? D / VEC : D)) return;
   const int per = (rows + gridDim.y - 1) / gridDim.y;
   const int t0 = blockIdx.y * per;
   const int t1 = t0 + per < rows ? t0 + per : rows;
-  float acc = 0.f;
-  for (int t = t0; t < t1; ++t)
-    acc += Elem<T>::load(dy + (size_t)t * D + j) * Elem<T>::load(x + (size_t)t * D + j) * rstd[t];
-  partial[(size_t)blockIdx.y * D + j] = acc;
+  float* out = partial + (size_t)blockIdx.y * D;
+  if (vec) {
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+#pragma unroll 4
+    for (int t = t0; t < t1; ++t) {
+      const u32x4 xv = *reinterpret_cast<const u32x4*>(x + (size_t)t * D + c * VEC);
+      const u32x4 gv = *reinterpret_cast<const u32x4*>(dy + (size_t)t * D + c * VEC);
+      const float r = rstd[t];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if constexpr (sizeof(T) == 2) {
+          acc[2 * j] += __uint_as_float(gv[j] << 16) * __uint_as_float(xv[j] << 16) * r;
+          acc[2 * j + 1] += __uint_as_float(gv[j] & 0xffff0000u) * __uint_as_float(xv[j] & 0xffff0000u) * r;
+        } else {
+          acc[j] += __uint_as_float(gv[j]) * __uint_as_float(xv[j]) * r;
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) out[c * VEC + j] = acc[j];
+  } else {
+    float acc = 0.f;
+    for (int t = t0; t < t1; ++t)
+      acc += Elem<T>::load(dy + (size_t)t * D + c) * Elem<T>::load(x + (size_t)t * D + c) * rstd[t];
+    out[c] = acc;
+  }
 }
 
-// Second half: the slabs added in ascending order, one rounding.
+// Second half: a block owns 32 columns; its eight groups of 32 threads add every eighth slab in
+// ascending order, then the eight sums are added in order.  One rounding.
 template <typename T>
 __global__ __launch_bounds__(256) void rms_norm_backward_weight_sum_kernel(
     const float* __restrict__ partial, int slabs, int D, T* __restrict__ dw) {
-  const int j = blockIdx.x * 256 + threadIdx.x;
-  if (j >= D) return;
+  __shared__ float s_sum[8][32];
+  const int col = blockIdx.x * 32 + (threadIdx.x & 31), grp = threadIdx.x >> 5;
   float acc = 0.f;
-  for (int s = 0; s < slabs; ++s) acc += partial[(size_t)s * D + j];
-  Elem<T>::store(dw + j, acc);
+  if (col < D) {
+#pragma unroll 8
+    for (int s = grp; s < slabs; s += 8) acc += partial[(size_t)s * D + col];
+  }
+  s_sum[grp][threadIdx.x & 31] = acc;
+  __syncthreads();
+  if (grp == 0 && col < D) {
+    float total = 0.f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) total += s_sum[q][threadIdx.x];
+    Elem<T>::store(dw + col, total);
+  }
 }
 
 // --------------------------------------------------------------------------------- router backward
@@ -777,10 +815,10 @@ extern "C" int fs2moe_router_backward(const float* logits, const int32_t* topk_i
   return check_launch("router_backward");
 }
 
-// slabs of rows for the weight gradient of the normalisation: at least 32 rows each, at most 64
+// slabs of rows for the weight gradient of the normalisation: at least 32 rows each, at most 256
 static int norm_weight_slabs(int64_t rows) {
   const int64_t s = rows / 32;
-  return s < 1 ? 1 : (s > 64 ? 64 : (int)s);
+  return s < 1 ? 1 : (s > 256 ? 256 : (int)s);
 }
 
 extern "C" int64_t fs2moe_rms_norm_backward_workspace_bytes(int32_t T, int32_t D) {
@@ -831,18 +869,21 @@ extern "C" int fs2moe_rms_norm_backward(const void* x, const void* weight, float
   if (dweight == nullptr) return FS2MOE_OK;
   // (with no rows the one slab sums nothing and the gradient is zero)
   const int slabs = norm_weight_slabs(T);
-  const dim3 grid((unsigned)((D + 255) / 256), (unsigned)slabs);
+  const int vec = dtype == FS2MOE_BF16 ? 8 : 4;
+  const int owners = D % vec == 0 ? D / vec : D;  // threads per slab
+  const dim3 grid((unsigned)((owners + 255) / 256), (unsigned)slabs);
+  const unsigned sum_blocks = (unsigned)((D + 31) / 32);
   if (dtype == FS2MOE_BF16) {
     hipLaunchKernelGGL(rms_norm_backward_weight_kernel<uint16_t>, grid, dim3(256), 0, st,
                        static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(dy), rstd, T, D,
                        partial);
-    hipLaunchKernelGGL(rms_norm_backward_weight_sum_kernel<uint16_t>, dim3(grid.x), dim3(256), 0, st,
+    hipLaunchKernelGGL(rms_norm_backward_weight_sum_kernel<uint16_t>, dim3(sum_blocks), dim3(256), 0, st,
                        partial, slabs, D, static_cast<uint16_t*>(dweight));
   } else {
     hipLaunchKernelGGL(rms_norm_backward_weight_kernel<float>, grid, dim3(256), 0, st,
                        static_cast<const float*>(x), static_cast<const float*>(dy), rstd, T, D,
                        partial);
-    hipLaunchKernelGGL(rms_norm_backward_weight_sum_kernel<float>, dim3(grid.x), dim3(256), 0, st,
+    hipLaunchKernelGGL(rms_norm_backward_weight_sum_kernel<float>, dim3(sum_blocks), dim3(256), 0, st,
                        partial, slabs, D, static_cast<float*>(dweight));
   }
   return check_launch("rms_norm_backward (weight)");

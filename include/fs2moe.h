@@ -367,7 +367,7 @@ int fs2moe_router_backward(const float* logits, const int32_t* topk_idx, const f
  * torch.nn.functional.rms_norm (nn/normalization.py:234-236), the ffn_layer_norm call of
  * models/transformer_lm/decoder_layer.py:187-191.
  *   dx[t] = r_t * (dy[t] * weight) - x[t] * r_t^3 * <dy[t] * weight, x[t]> / D
- *   dweight[j] = sum over t (ascending, in up to 64 slabs) of dy[t, j] * x[t, j] * r_t
+ *   dweight[j] = sum over t (ascending, in up to 256 slabs) of dy[t, j] * x[t, j] * r_t
  * all in f32 with one rounding per stored element.
  *   x, dy [T, D] dtype   weight [D] dtype or NULL   dx [T, D] dtype (out; must not alias x or dy)
  *   dweight [D] dtype (out) or NULL; when given, workspace must hold
