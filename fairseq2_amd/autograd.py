@@ -37,6 +37,84 @@ from torch import Tensor
 from fairseq2_amd import _abi
 
 
+def experts_forward(xe, counts, offsets, wg, wu, wd, e, act=None):
+    """``(ye, g, u)`` of the grouped experts on the rows ``xe``.  Where the expert kernel can, it
+    leaves the gate and the up product behind for the backward pass (what autograd would save);
+    otherwise ``g`` and ``u`` are None and :func:`experts_backward` computes them again."""
+    if act is not None:
+        # a gate activation other than SiLU (experts.py:84-87 takes any module): the module's own
+        # forward between the library's plain grouped GEMMs, in f32 with one rounding
+        grp = dict(counts=counts, offsets=offsets, num_experts=e)
+        g = _abi.grouped_gemm(xe, wg, _abi.W_IN_OUT, **grp)
+        u = _abi.grouped_gemm(xe, wu, _abi.W_IN_OUT, **grp)
+        h = (act(g.float()) * u.float()).to(xe.dtype)
+        return _abi.grouped_gemm(h, wd, _abi.W_IN_OUT, **grp), g, u
+    if _abi.keeps_products(xe.shape[1], wd.shape[0] // e, xe.shape[0], xe.dtype):
+        ye, _, g, u = _abi.grouped_swiglu_keep(xe, counts, offsets, wg, wu, wd, e)
+        return ye, g, u
+    return _abi.grouped_swiglu(xe, counts, offsets, wg, wu, wd, e)[0], None, None
+
+
+def dense_forward(x, sg, su, sd):
+    """``(y, g, u)`` of the shared expert (``nn.Linear``-oriented weights); ``g``, ``u`` as above."""
+    if _abi.keeps_products(x.shape[1], sg.shape[0], x.shape[0], x.dtype):
+        return _abi.dense_swiglu_keep(x, sg, su, sd)
+    return _abi.dense_swiglu(x, sg, su, sd), None, None
+
+
+def experts_backward(xe, dye, wg, wu, wd, g, u, e, counts, offsets, act, need_w):
+    """``(dxe_g, dxe_u, d_wg, d_wu, d_wd)`` of the grouped experts: the input gradient as one
+    tensor (``dxe_u`` None) where the two-source kernel runs, else as the two products whose sum it
+    is; weight gradients None where ``need_w`` (gate, up, down) says so."""
+    IN_OUT, OUT_IN = _abi.W_IN_OUT, _abi.W_OUT_IN
+    grp = dict(counts=counts, offsets=offsets, num_experts=e)
+    dh = _abi.grouped_gemm(dye, wd, OUT_IN, **grp)
+    if act is not None:
+        # the module's own derivative, through torch.autograd on its forward (f32, one rounding)
+        with torch.enable_grad():
+            g32 = g.float().requires_grad_(True)
+            a32 = act(g32)
+        u32, dh32 = u.float(), dh.float()
+        (dg32,) = torch.autograd.grad(a32, g32, dh32 * u32)
+        a32 = a32.detach()
+        h, dg, du = (a32 * u32).to(xe.dtype), dg32.to(xe.dtype), (dh32 * a32).to(xe.dtype)
+    elif g is None:
+        g = _abi.grouped_gemm(xe, wg, IN_OUT, **grp)
+        u = _abi.grouped_gemm(xe, wu, IN_OUT, **grp)
+        h, dg, du = _abi.swiglu_backward(g, u, dh)  # in place over g and u
+    else:
+        h, dg, du = _abi.swiglu_backward(g, u, dh, in_place=False)  # g, u are autograd's to keep
+    d_wd = _abi.grouped_wgrad(h, dye, **grp) if need_w[2] else None
+    d_wg = _abi.grouped_wgrad(xe, dg, **grp) if need_w[0] else None
+    d_wu = _abi.grouped_wgrad(xe, du, **grp) if need_w[1] else None
+    # dxe = dg @ Wg^T + du @ Wu^T: one kernel and one rounding where the library has it, else the
+    # two products apart (their sum is then taken where dxe is used)
+    if _abi.grouped_gemm_sum_supported(dg.shape[1], xe.shape[1], dg.shape[0], dg.dtype):
+        dxe_g, dxe_u = _abi.grouped_gemm_sum(dg, wg, du, wu, **grp), None
+    else:
+        dxe_g = _abi.grouped_gemm(dg, wg, OUT_IN, **grp)
+        dxe_u = _abi.grouped_gemm(du, wu, OUT_IN, **grp)
+    return dxe_g, dxe_u, d_wg, d_wu, d_wd
+
+
+def dense_backward(x, dout, sg, su, sd, g_s, u_s, need_w, need_x):
+    """``(dx_parts, d_sg, d_su, d_sd)`` of the shared expert: the input gradient as the two
+    products whose sum it is (an empty list unless ``need_x``)."""
+    IN_OUT, OUT_IN = _abi.W_IN_OUT, _abi.W_OUT_IN
+    dh_s = _abi.grouped_gemm(dout, sd, IN_OUT)
+    if g_s is None:
+        g_s = _abi.grouped_gemm(x, sg, OUT_IN)
+        u_s = _abi.grouped_gemm(x, su, OUT_IN)
+        h_s, dg_s, du_s = _abi.swiglu_backward(g_s, u_s, dh_s)
+    else:
+        h_s, dg_s, du_s = _abi.swiglu_backward(g_s, u_s, dh_s, in_place=False)
+    d_sd = _abi.grouped_wgrad(dout, h_s) if need_w[2] else None
+    d_sg = _abi.grouped_wgrad(dg_s, x) if need_w[0] else None
+    d_su = _abi.grouped_wgrad(du_s, x) if need_w[1] else None
+    parts = [_abi.grouped_gemm(dg_s, sg, IN_OUT), _abi.grouped_gemm(du_s, su, IN_OUT)] if need_x else []
+    return parts, d_sg, d_su, d_sd
+
+
 def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg, norm_w=None):
     """The staged forward pass; returns ``(out, saved)`` with what :func:`backward_from` needs.
     With ``cfg["norm_eps"]`` set the rows are RMS-normalised (weight ``norm_w`` or none) on the way
@@ -49,28 +127,10 @@ def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg, norm_w=None
     else:
         idx, w, logits = _abi.router_topk(x, router, cfg["router_bias"], k, score_fn, renorm, want_logits=True)
     disp = _abi.dispatch(idx, w, x, e, tile_m, scale_input, gather=True)
-    # where the expert kernel can, it leaves the gate and the up product behind for the backward
-    # pass (what autograd would save); otherwise backward_from computes them again
-    g = u = None
-    act = cfg.get("activation")
-    if act is not None:
-        # a gate activation other than SiLU (experts.py:84-87 takes any module): the module's own
-        # forward between the library's plain grouped GEMMs, in f32 with one rounding
-        grp = dict(counts=disp.counts, offsets=disp.offsets, num_experts=e)
-        g = _abi.grouped_gemm(disp.xe, wg, _abi.W_IN_OUT, **grp)
-        u = _abi.grouped_gemm(disp.xe, wu, _abi.W_IN_OUT, **grp)
-        h = (act(g.float()) * u.float()).to(x.dtype)
-        ye = _abi.grouped_gemm(h, wd, _abi.W_IN_OUT, **grp)
-    elif _abi.keeps_products(x.shape[1], wd.shape[0] // e, disp.xe.shape[0], x.dtype):
-        ye, _, g, u = _abi.grouped_swiglu_keep(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
-    else:
-        ye, _ = _abi.grouped_swiglu(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e)
+    ye, g, u = experts_forward(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e, cfg.get("activation"))
     base = g_s = u_s = None
     if sg is not None:
-        if _abi.keeps_products(x.shape[1], sg.shape[0], x.shape[0], x.dtype):
-            base, g_s, u_s = _abi.dense_swiglu_keep(x, sg, su, sd)
-        else:
-            base = _abi.dense_swiglu(x, sg, su, sd)
+        base, g_s, u_s = dense_forward(x, sg, su, sd)
     out = _abi.combine(ye, disp.inv_perm, idx, w, base, not scale_input, out=base, residual=residual)
     xn = x if cfg.get("norm_eps") is not None else None
     return out, (idx, w, logits, disp.counts, disp.offsets, disp.inv_perm, disp.xe, ye, g, u, g_s, u_s, xn)
@@ -83,39 +143,13 @@ def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
     e, tile_m = cfg["num_experts"], cfg["tile_m"]
     score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
     dout = dout.contiguous()
-    IN_OUT, OUT_IN = _abi.W_IN_OUT, _abi.W_OUT_IN
-    grp = dict(counts=counts, offsets=offsets, num_experts=e)
+    OUT_IN = _abi.W_OUT_IN
 
     # output gradients in expert order (times the combine weight when it scales the output);
     # the permutation is the forward pass's: dispatch is deterministic
     dye = _abi.dispatch(idx, w, dout, e, tile_m, not scale_input, gather=True).xe
-    dh = _abi.grouped_gemm(dye, wd, OUT_IN, **grp)
-    act = cfg.get("activation")
-    if act is not None:
-        # the module's own derivative, through torch.autograd on its forward (f32, one rounding)
-        with torch.enable_grad():
-            g32 = g.float().requires_grad_(True)
-            a32 = act(g32)
-        u32, dh32 = u.float(), dh.float()
-        (dg32,) = torch.autograd.grad(a32, g32, dh32 * u32)
-        a32 = a32.detach()
-        h, dg, du = (a32 * u32).to(x.dtype), dg32.to(x.dtype), (dh32 * a32).to(x.dtype)
-    elif g is None:
-        g = _abi.grouped_gemm(xe, wg, IN_OUT, **grp)
-        u = _abi.grouped_gemm(xe, wu, IN_OUT, **grp)
-        h, dg, du = _abi.swiglu_backward(g, u, dh)  # in place over g and u
-    else:
-        h, dg, du = _abi.swiglu_backward(g, u, dh, in_place=False)  # g, u are autograd's to keep
-    d_wd = _abi.grouped_wgrad(h, dye, **grp) if need[4] else None
-    d_wg = _abi.grouped_wgrad(xe, dg, **grp) if need[2] else None
-    d_wu = _abi.grouped_wgrad(xe, du, **grp) if need[3] else None
-    # dxe = dg @ Wg^T + du @ Wu^T: one kernel and one rounding where the library has it, else the
-    # two products apart (their sum is then taken where dxe is used)
-    if _abi.grouped_gemm_sum_supported(dg.shape[1], x.shape[1], dg.shape[0], dg.dtype):
-        dxe_g, dxe_u = _abi.grouped_gemm_sum(dg, wg, du, wu, **grp), None
-    else:
-        dxe_g = _abi.grouped_gemm(dg, wg, OUT_IN, **grp)
-        dxe_u = _abi.grouped_gemm(du, wu, OUT_IN, **grp)
+    dxe_g, dxe_u, d_wg, d_wu, d_wd = experts_backward(
+        xe, dye, wg, wu, wd, g, u, e, counts, offsets, cfg.get("activation"), need[2:5])
 
     # combine weights -> logits -> router and x
     if scale_input:
@@ -134,18 +168,8 @@ def backward_from(x, router, wg, wu, wd, sg, su, sd, saved, cfg, dout, need):
 
     d_sg = d_su = d_sd = None
     if sg is not None:
-        dh_s = _abi.grouped_gemm(dout, sd, IN_OUT)
-        if g_s is None:
-            g_s = _abi.grouped_gemm(x, sg, OUT_IN)
-            u_s = _abi.grouped_gemm(x, su, OUT_IN)
-            h_s, dg_s, du_s = _abi.swiglu_backward(g_s, u_s, dh_s)
-        else:
-            h_s, dg_s, du_s = _abi.swiglu_backward(g_s, u_s, dh_s, in_place=False)
-        d_sd = _abi.grouped_wgrad(dout, h_s) if need[7] else None
-        d_sg = _abi.grouped_wgrad(dg_s, x) if need[5] else None
-        d_su = _abi.grouped_wgrad(du_s, x) if need[6] else None
-        if need[0]:
-            dx_parts += [_abi.grouped_gemm(dg_s, sg, IN_OUT), _abi.grouped_gemm(du_s, su, IN_OUT)]
+        parts, d_sg, d_su, d_sd = dense_backward(x, dout, sg, su, sd, g_s, u_s, need[5:8], need[0])
+        dx_parts += parts
 
     dx = None
     if need[0]:
@@ -192,3 +216,48 @@ class MoEFunction(torch.autograd.Function):
                 dx = None
         d_res = dout if ctx.has_residual and n[1] else None
         return dx, d_res, d_router, d_wg, d_wu, d_wd, d_sg, d_su, d_sd, d_norm_w, None
+
+
+def _sum_rounded_once(a: Tensor, b: Tensor | None) -> Tensor:
+    return a if b is None else (a.float() + b.float()).to(a.dtype)
+
+
+class GroupedExpertsFunction(torch.autograd.Function):
+    """The grouped experts alone, ``forward(xe, counts, offsets, wg, wu, wd, e, act)`` -> ``ye``: what
+    :class:`fairseq2_amd.moe.GroupedExpertNetwork` runs when called by itself in training
+    (``experts.py:201-213``)."""
+
+    @staticmethod
+    def forward(ctx, xe, counts, offsets, wg, wu, wd, e, act):  # noqa: D102
+        ye, g, u = experts_forward(xe, counts, offsets, wg, wu, wd, e, act)
+        ctx.e, ctx.act = e, act
+        ctx.save_for_backward(xe, counts, offsets, wg, wu, wd, g, u)
+        return ye
+
+    @staticmethod
+    @torch.no_grad()
+    def backward(ctx, dye):  # noqa: D102
+        xe, counts, offsets, wg, wu, wd, g, u = ctx.saved_tensors
+        n = ctx.needs_input_grad
+        dxe_g, dxe_u, d_wg, d_wu, d_wd = experts_backward(
+            xe, dye.contiguous(), wg, wu, wd, g, u, ctx.e, counts, offsets, ctx.act, n[3:6])
+        return (_sum_rounded_once(dxe_g, dxe_u) if n[0] else None), None, None, d_wg, d_wu, d_wd, None, None
+
+
+class DenseSwiGLUFunction(torch.autograd.Function):
+    """The shared expert alone, ``forward(x, sg, su, sd)`` -> ``y`` with ``nn.Linear``-oriented
+    weights: :class:`fairseq2_amd.moe.GLUFeedForwardNetwork` in training (``ffn.py:374-395``)."""
+
+    @staticmethod
+    def forward(ctx, x, sg, su, sd):  # noqa: D102
+        y, g, u = dense_forward(x, sg, su, sd)
+        ctx.save_for_backward(x, sg, su, sd, g, u)
+        return y
+
+    @staticmethod
+    @torch.no_grad()
+    def backward(ctx, dy):  # noqa: D102
+        x, sg, su, sd, g, u = ctx.saved_tensors
+        n = ctx.needs_input_grad
+        parts, d_sg, d_su, d_sd = dense_backward(x, dy.contiguous(), sg, su, sd, g, u, n[1:4], n[0])
+        return (_sum_rounded_once(*parts) if n[0] else None), d_sg, d_su, d_sd

@@ -204,7 +204,9 @@ class GroupedExpertNetwork(ExpertNetwork):
         self, xe: Tensor, counts: Tensor, offsets: Tensor, row_map: Tensor | None = None
     ) -> Tensor:
         """Runs every expert on its block of rows of ``xe`` (rows, D); with ``row_map``, row ``r``
-        is ``xe[row_map[r]]`` and ``xe`` is the token matrix."""
+        is ``xe[row_map[r]]`` and ``xe`` is the token matrix.  Inference only (the training
+        paths are :meth:`forward` and the layer's)."""
+        _require_forward_only(xe, self.gate_proj, self.inner_proj, self.output_proj)
         if not self.has_fused_gate:
             # experts.py:107-112 with the module's own activation between the library's GEMMs
             if self.has_fp8_weights or row_map is not None:
@@ -232,11 +234,25 @@ class GroupedExpertNetwork(ExpertNetwork):
         """The reference's dense calling convention: every expert gets the same
         number of rows (``experts.py:201-213``)."""
         _require_device(x)
-        _require_forward_only(x, self.gate_proj, self.inner_proj, self.output_proj)
         e, n, d = x.shape
         if e != self.num_local_experts or d != self.model_dim:
             raise ValueError(f"expected ({self.num_local_experts}, *, {self.model_dim}), got {tuple(x.shape)}")
         counts, offsets = self._uniform_groups(n, x.device)
+        params = (self.gate_proj, self.inner_proj, self.output_proj)
+        if torch.is_grad_enabled() and any(t.requires_grad for t in (x, *params)):
+            # training: the experts alone as one autograd function on the library's backward kernels
+            if self.has_fp8_weights:
+                raise RuntimeError("fairseq2_amd: e4m3 expert weights are an inference format")
+            if not self.has_fused_gate and any(p.requires_grad for p in self.activation.parameters()):
+                raise RuntimeError("fairseq2_amd: a gate activation with parameters of its own is not differentiated")
+            if n == 0:
+                return torch.empty_like(x)
+            from fairseq2_amd.autograd import GroupedExpertsFunction
+
+            ye = GroupedExpertsFunction.apply(
+                x.reshape(e * n, d).contiguous(), counts, offsets, *params, e,
+                None if self.has_fused_gate else self.activation)
+            return ye.view(e, n, d)
         return self.forward_rows(x.reshape(e * n, d).contiguous(), counts, offsets).view(e, n, d)
 
     def _uniform_groups(self, n: int, device: torch.device) -> tuple[Tensor, Tensor]:
@@ -307,10 +323,15 @@ class GLUFeedForwardNetwork(FeedForwardNetwork):
 
     def forward(self, seqs: Tensor) -> Tensor:
         _require_device(seqs)
-        _require_forward_only(
-            seqs, self.gate_proj.weight, self.inner_proj.weight, self.output_proj.weight
-        )
         x = seqs.reshape(-1, seqs.shape[-1]).contiguous()
+        params = (self.gate_proj.weight, self.inner_proj.weight, self.output_proj.weight)
+        if torch.is_grad_enabled() and any(t.requires_grad for t in (seqs, *params)):
+            # training: one autograd function on the library's backward kernels
+            if x.shape[0] == 0:
+                return torch.empty_like(seqs)
+            from fairseq2_amd.autograd import DenseSwiGLUFunction
+
+            return DenseSwiGLUFunction.apply(x, *params).view(seqs.shape)
         y = _abi.dense_swiglu(
             x, self.gate_proj.weight.detach(), self.inner_proj.weight.detach(),
             self.output_proj.weight.detach(),

@@ -547,6 +547,80 @@ def test_gradients_through_the_normalisation_compose(gpu_device, dtype):
     torch.testing.assert_close(got_x.float(), want_x.float(), rtol=2 ** -7 if dtype == "bf16" else 1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("e,n,d,f,act", [(6, 37, 128, 192, None), (4, 300, 256, 128, None), (3, 50, 72, 40, None),
+                                         (4, 64, 128, 64, "gelu")])
+def test_grouped_expert_network_alone_is_differentiable(gpu_device, dtype, e, n, d, f, act):
+    """``GroupedExpertNetwork.forward((E, n, D))`` (``experts.py:201-213``) under autograd: the
+    gradients of its input and of the three weights against float64 autograd through the oracle's
+    expert, and the training call's values are the inference call's."""
+    from fairseq2_amd.moe import GroupedExpertNetwork
+
+    td = TORCH_DTYPE[dtype]
+    gen = torch.Generator().manual_seed(e * 100 + n)
+    activation = torch.nn.GELU(approximate="tanh") if act else None
+    net = GroupedExpertNetwork(e, d, f, activation=activation, device=gpu_device, dtype=td)
+    wg = (0.08 * torch.randn(e * d, f, generator=gen)).to(td)
+    wu = (0.08 * torch.randn(e * d, f, generator=gen)).to(td)
+    wd = (0.08 * torch.randn(e * f, d, generator=gen)).to(td)
+    net.load_state_dict({"gate_proj": wg, "inner_proj": wu, "output_proj": wd})
+    x = torch.randn(e, n, d, generator=gen).to(td)
+    dy = torch.randn(e, n, d, generator=gen).to(td)
+    c = lambda t: t.double().clone().requires_grad_(True)  # noqa: E731
+    x64, wg64, wu64, wd64 = c(x), c(wg), c(wu), c(wd)
+    fn = torch.nn.functional.silu if activation is None else activation
+    ref = torch.stack([(fn(x64[i] @ wg64.view(e, d, f)[i]) * (x64[i] @ wu64.view(e, d, f)[i])) @ wd64.view(e, f, d)[i]
+                       for i in range(e)])
+    if activation is None:  # the same thing as the oracle states it
+        torch.testing.assert_close(ref[0], O.glu_expert(x64[0], wg64.view(e, d, f)[0], wu64.view(e, d, f)[0],
+                                                        wd64.view(e, f, d)[0]))
+    ref.backward(dy.double())
+    xd = x.to(gpu_device).requires_grad_(True)
+    y = net(xd)
+    with torch.no_grad():
+        assert torch.equal(y, net(xd))
+    y.backward(dy.to(gpu_device))
+    assert_grad_close(xd.grad, x64.grad, dtype, "d x")
+    assert_grad_close(net.gate_proj.grad, wg64.grad, dtype, "d gate_proj")
+    assert_grad_close(net.inner_proj.grad, wu64.grad, dtype, "d inner_proj")
+    assert_grad_close(net.output_proj.grad, wd64.grad, dtype, "d output_proj")
+    # frozen weights: only the input's gradient, the same bits
+    net.requires_grad_(False)
+    x2 = x.to(gpu_device).requires_grad_(True)
+    net(x2).backward(dy.to(gpu_device))
+    assert torch.equal(x2.grad, xd.grad) and net.gate_proj.grad is not None
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("shape,d,f", [((2, 37), 128, 192), ((700,), 256, 128), ((3, 5, 7), 72, 40)])
+def test_glu_feed_forward_network_alone_is_differentiable(gpu_device, dtype, shape, d, f):
+    """``GLUFeedForwardNetwork.forward`` (``ffn.py:374-395``) under autograd, against float64
+    autograd through the oracle's shared expert."""
+    from fairseq2_amd.moe import GLUFeedForwardNetwork
+
+    td = TORCH_DTYPE[dtype]
+    gen = torch.Generator().manual_seed(d + f)
+    net = GLUFeedForwardNetwork(d, f, inner_dim_scale=1.0, device=gpu_device, dtype=td)
+    sg = (0.08 * torch.randn(f, d, generator=gen)).to(td)
+    su = (0.08 * torch.randn(f, d, generator=gen)).to(td)
+    sd = (0.08 * torch.randn(d, f, generator=gen)).to(td)
+    net.load_state_dict({"gate_proj.weight": sg, "inner_proj.weight": su, "output_proj.weight": sd})
+    x = torch.randn(*shape, d, generator=gen).to(td)
+    dy = torch.randn(*shape, d, generator=gen).to(td)
+    c = lambda t: t.double().clone().requires_grad_(True)  # noqa: E731
+    x64, sg64, su64, sd64 = c(x), c(sg), c(su), c(sd)
+    O.shared_glu(x64, sg64, su64, sd64).backward(dy.double())
+    xd = x.to(gpu_device).requires_grad_(True)
+    y = net(xd)
+    with torch.no_grad():
+        assert torch.equal(y, net(xd))
+    y.backward(dy.to(gpu_device))
+    assert_grad_close(xd.grad, x64.grad, dtype, "d x")
+    assert_grad_close(net.gate_proj.weight.grad, sg64.grad, dtype, "d gate_proj")
+    assert_grad_close(net.inner_proj.weight.grad, su64.grad, dtype, "d inner_proj")
+    assert_grad_close(net.output_proj.weight.grad, sd64.grad, dtype, "d output_proj")
+
+
 def test_frozen_parameters_get_no_gradient_and_unsupported_cases_say_so(gpu_device):
     wl = W.make_workload_from_spec(W.small_spec(dtype="bf16", tokens=64, num_experts=8, inner_dim=128, seed=3))
     m = build_module(wl, gpu_device)  # frozen
