@@ -194,6 +194,76 @@ def test_full_size_weight_gradient_and_kept_products(gpu_device):
         assert_grad_close(up[sl], ref.double().cpu(), "bf16", f"up product of expert {ex}")
 
 
+@pytest.mark.parametrize("name", ["mixtral_8x7b", "llama4_scout"])
+def test_full_size_training_step_of_the_other_shapes(gpu_device, name):
+    """One training step of the module at the Mixtral and the Llama-4 Scout prefill shapes (8192
+    tokens): the weight gradients of sampled experts, and of the shared expert, against the chain
+    rule spelled out in torch f32 on the same device from the module's own routing
+    (``moe.py:131-150``, ``experts.py:107-112``); every gradient finite, an expert without tokens
+    with none.  The values of the training forward are the inference path's."""
+    import torch.nn.functional as F
+
+    wl = W.make_workload(name)
+    s = wl.spec
+    dev = gpu_device
+    d, f, e, k = s.model_dim, s.inner_dim, s.num_experts, s.top_k
+    m = build_module(wl, dev).train().requires_grad_(True)
+    x = wl.x.to(torch.bfloat16).to(dev).requires_grad_(True)
+    gen = torch.Generator().manual_seed(13)
+    dout = torch.randn(wl.x.shape, generator=gen).to(torch.bfloat16).to(dev)
+    out = m(x)
+    with torch.no_grad():
+        assert torch.equal(out, m(x))
+    out.backward(dout)
+    torch.cuda.synchronize()
+    for n_, p_ in m.named_parameters():
+        assert p_.grad is not None and bool(torch.isfinite(p_.grad).all()), n_
+    assert bool(torch.isfinite(x.grad).all())
+    rows, g2 = x.detach().reshape(-1, d), dout.reshape(-1, d)
+    idx, w, _ = _abi.router_topk(rows, m.router.detach(), m.router_bias, k, _abi.SCORE_SOFTMAX
+                                 if s.mode.score_fn == "softmax" else _abi.SCORE_SIGMOID, s.mode.renormalize)
+    counts = torch.bincount(idx.flatten().long(), minlength=e).cpu()
+    order = torch.argsort(counts, descending=True)
+    scale_in = s.mode.scale_on == "input"
+    bf = lambda t: t.to(torch.bfloat16).float()  # noqa: E731
+    for ex in {int(order[0]), int(order[e // 2]), int(order[-1])}:
+        sel = idx == ex
+        tok = sel.any(dim=1).nonzero().squeeze(1)
+        wg, wu, wd = (p_.detach().view(e, -1, p_.shape[1])[ex].float()
+                      for p_ in (m.experts.gate_proj, m.experts.inner_proj, m.experts.output_proj))
+        got = [p_.grad.view(e, -1, p_.shape[1])[ex]
+               for p_ in (m.experts.gate_proj, m.experts.inner_proj, m.experts.output_proj)]
+        _say(f"  {name}: expert {ex}, {tok.numel()} tokens")
+        if tok.numel() == 0:
+            assert not any(bool(t.any()) for t in got)
+            continue
+        we = (w * sel).sum(dim=1)[tok][:, None]
+        xe = bf(rows[tok].float() * we) if scale_in else rows[tok].float()
+        dye = g2[tok].float() if scale_in else bf(g2[tok].float() * we)
+        gate, up = bf(xe @ wg), bf(xe @ wu)
+        sig = torch.sigmoid(gate)
+        h = bf(F.silu(gate) * up)
+        dh = bf(dye @ wd.t())
+        dg = bf(dh * up * (sig * (1 + gate * (1 - sig))))
+        du = bf(dh * F.silu(gate))
+        for what, got_t, ref in (("gate_proj", got[0], xe.t() @ dg), ("inner_proj", got[1], xe.t() @ du),
+                                 ("output_proj", got[2], h.t() @ dye)):
+            assert_grad_close(got_t, ref.double().cpu(), "bf16", f"{name}: d {what} of expert {ex}")
+    if s.shared:
+        se = m.shared_expert
+        sg, su, sd = (p_.weight.detach().float() for p_ in (se.gate_proj, se.inner_proj, se.output_proj))
+        xf, gf = rows.float(), g2.float()
+        gate, up = bf(xf @ sg.t()), bf(xf @ su.t())
+        sig = torch.sigmoid(gate)
+        h = bf(F.silu(gate) * up)
+        dh = bf(gf @ sd)
+        dg = bf(dh * up * (sig * (1 + gate * (1 - sig))))
+        du = bf(dh * F.silu(gate))
+        assert_grad_close(se.output_proj.weight.grad, (gf.t() @ h).double().cpu(), "bf16", f"{name}: d shared output_proj")
+        assert_grad_close(se.gate_proj.weight.grad, (dg.t() @ xf).double().cpu(), "bf16", f"{name}: d shared gate_proj")
+        assert_grad_close(se.inner_proj.weight.grad, (du.t() @ xf).double().cpu(), "bf16", f"{name}: d shared inner_proj")
+
+
 def test_dense_swiglu_keep_leaves_the_two_products(gpu_device):
     """The shared expert's training forward: ``y`` as the inference kernel gives it, bit for bit, and
     the two products as two GEMMs give them."""
