@@ -30,6 +30,8 @@ namespace wgk {
 constexpr int TM = 256, TN = 256, WAVES = 8;
 constexpr int SMEM_BYTES = 65536;  // two chunks of both operands
 }
+// what a load past the end of an operand reads
+__device__ __attribute__((aligned(16))) uint32_t kZero16[4] = {0u, 0u, 0u, 0u};  // (not const: a global address, so the loads stay global loads)
 
 // MAPPED: A's rows are read through a_map.  A template parameter, not a test of the pointer: behind
 // a condition the map entry's load is waited for with every other load of the wave (the counter
@@ -99,14 +101,13 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
-  // Loads are unconditional, from clamped addresses (a select behind a load would make the wave wait
-  // for it at once); what lies past the expert's rows or the matrix's columns is zeroed when the
-  // registers go to LDS.
+  // Loads are unconditional; what lies past the expert's rows or the matrix's columns is read from
+  // 16 zero bytes instead (the address is selected, not the data: any instruction on the loaded
+  // registers other than the LDS store gets scheduled early and waits for the load there).
   // Two sets of registers, so that two chunks are on their way from memory at any time (one chunk's
   // loads take about as long as its MFMAs do: with a single set every chunk waited for its loads).
   u32x4 ra[2][PER_THREAD], rb[2][PER_THREAD];
-  bool va[2][PER_THREAD], vb[2][PER_THREAD];
-  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  const T* zero_src = reinterpret_cast<const T*>(kZero16);
   auto load_chunk = [&](auto set_c, int r0) {
     constexpr int set = decltype(set_c)::value;
     int rr[PER_THREAD], arow[PER_THREAD];
@@ -125,13 +126,11 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
       const int c = tid + WAVES * 64 * i;
       const int k = c / ROW_CHUNKS, ch = c % ROW_CHUNKS;
       const bool row_ok = r0 + k < cnt;
-      const bool a_ok = m0 + ch * VEC < M, b_ok = n0 + ch * VEC < N;
-      va[set][i] = row_ok && a_ok;
-      vb[set][i] = row_ok && b_ok;
-      ra[set][i] =
-          *reinterpret_cast<const u32x4*>(A + (size_t)arow[i] * lda + (a_ok ? m0 + ch * VEC : 0));
-      rb[set][i] =
-          *reinterpret_cast<const u32x4*>(B + (size_t)rr[i] * ldb + (b_ok ? n0 + ch * VEC : 0));
+      const bool a_ok = row_ok && m0 + ch * VEC < M, b_ok = row_ok && n0 + ch * VEC < N;
+      const T* pa = a_ok ? A + (size_t)arow[i] * lda + m0 + ch * VEC : zero_src;
+      const T* pb = b_ok ? B + (size_t)rr[i] * ldb + n0 + ch * VEC : zero_src;
+      ra[set][i] = *reinterpret_cast<const u32x4*>(pa);
+      rb[set][i] = *reinterpret_cast<const u32x4*>(pb);
     }
   };
   auto store_chunk = [&](auto set_c, int buf) {
@@ -145,8 +144,8 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
       // bf16: chunk ch of row k sits in slot ch ^ ((k & 3) << 2), so that the four consecutive rows
       // a transposing read touches lie 64 bytes apart
       const int slot = BF16 ? (ch ^ ((k & 3) << 2)) : ch;
-      *reinterpret_cast<u32x4*>(sA + k * ROWB + slot * 16) = va[set][i] ? ra[set][i] : zero4;
-      *reinterpret_cast<u32x4*>(sB + k * ROWB + slot * 16) = vb[set][i] ? rb[set][i] : zero4;
+      *reinterpret_cast<u32x4*>(sA + k * ROWB + slot * 16) = ra[set][i];
+      *reinterpret_cast<u32x4*>(sB + k * ROWB + slot * 16) = rb[set][i];
     }
   };
 
@@ -216,23 +215,28 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
   const int chunks = (cnt + RK - 1) / RK;
   using Set0 = std::integral_constant<int, 0>;
   using Set1 = std::integral_constant<int, 1>;
+  // Every load and store of the loop is unconditional (chunks past the last one load clamped rows
+  // and store zeros into the buffer nobody reads any more): behind a condition the compiler cannot
+  // count the loads in flight, and waits for all of them, the other set's included, before a store.
   if (chunks > 0) {
     load_chunk(Set0{}, 0);
-    if (chunks > 1) load_chunk(Set1{}, RK);
+    load_chunk(Set1{}, RK);
     store_chunk(Set0{}, 0);
-    if (chunks > 2) load_chunk(Set0{}, 2 * RK);
-    __syncthreads();
+    load_chunk(Set0{}, 2 * RK);
+    lds_barrier();
   }
   auto step = [&](int i, auto next_set) {
-    if (i + 1 < chunks) store_chunk(next_set, (i + 1) & 1);
-    if (i + 3 < chunks) load_chunk(next_set, (i + 3) * RK);
+    store_chunk(next_set, (i + 1) & 1);
+    load_chunk(next_set, (i + 3) * RK);
     compute_chunk(i & 1);
     lds_barrier();  // the loads of the next chunks stay in flight
   };
-  for (int i = 0; i < chunks; i += 2) {
-    step(i, Set1{});
-    if (i + 1 < chunks) step(i + 1, Set0{});
+  int ci = 0;
+  for (; ci + 1 < chunks; ci += 2) {
+    step(ci, Set1{});
+    step(ci + 1, Set0{});
   }
+  if (ci < chunks) step(ci, Set1{});
 
   // Accumulator layout: the lane holds row m = lr of fragment tm and columns 8 q + 4 lk + {0..3} of
   // fragment tn in registers 4 q .. 4 q + 3.
