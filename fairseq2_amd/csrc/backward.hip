@@ -18,16 +18,20 @@
 namespace fs2moe {
 
 // ---------------------------------------------------------------------------------- weight gradient
-// C_e [M, N] = sum over the rows r of expert e of A[r, :M]^T B[r, :N].  A block of 8 waves owns a
-// 256 x 256 tile of one expert's gradient (a wave 128 x 64: 4 x 2 MFMA tiles) and walks the expert's
-// rows RK at a time (32 for bf16, 16 for f32).  Both chunks go to LDS as they lie in memory (row =
-// contraction index, columns contiguous) and come back through the transposing LDS read (bf16) or
-// as single floats (f32), each already in MFMA operand order.  LDS holds two chunks: while one is
-// multiplied the next is written from registers and the two after that are on their way from memory
-// in two sets of registers, so there is one barrier per chunk, which orders LDS traffic only.  Rows
-// past the expert's count are zero-filled, experts without rows get a zero gradient.
+// C_e [M, N] = sum over the rows r of expert e of A[r, :M]^T B[r, :N].  A block owns a 256 x 256 tile
+// of one expert's gradient and walks the expert's rows RK at a time (32 for bf16, 16 for f32).  Eight
+// consumer waves multiply (a wave 128 x 64: 4 x 2 MFMA tiles); four producer waves, one per SIMD,
+// move the data: a wave that waits for memory issues nothing else, so loads issued by the waves that
+// multiply cost matrix-pipe time.  Both chunks go to LDS as they lie in memory (row = contraction
+// index, columns contiguous) and come back through the transposing LDS read (bf16) or as single
+// floats (f32), each already in MFMA operand order.  LDS holds two chunks: while one is multiplied
+// the producers write the next from registers and the two after that are on their way from memory
+// in two sets of registers, so there is one barrier per chunk, which orders LDS traffic only.
+// (Chunks of twice the rows, a half per register set and one barrier per chunk, were slower: 277
+// against 244 us on 8 experts of 8192 rows.)  Rows past the expert's count are zero-filled,
+// experts without rows get a zero gradient.
 namespace wgk {
-constexpr int TM = 256, TN = 256, WAVES = 8;
+constexpr int TM = 256, TN = 256, CONSUMERS = 8, PRODUCERS = 4, WAVES = CONSUMERS + PRODUCERS;
 constexpr int SMEM_BYTES = 65536;  // two chunks of both operands
 }
 // what a load past the end of an operand reads
@@ -46,7 +50,8 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
   constexpr int RK = BF16 ? 32 : 16;              // rows per chunk
   constexpr int VEC = 16 / sizeof(T);             // elements per 16-byte chunk
   constexpr int ROW_CHUNKS = TM / VEC;            // 16-byte chunks per LDS row (32 or 64)
-  constexpr int PER_THREAD = RK * ROW_CHUNKS / (WAVES * 64);  // chunks per thread and operand (2)
+  constexpr int PLANES = PRODUCERS * 64;          // lanes that move data
+  constexpr int PER_THREAD = RK * ROW_CHUNKS / PLANES;  // chunks per producer lane and operand (4)
   constexpr int ROWB = TM * sizeof(T);            // bytes per LDS row (512 or 1024)
   constexpr int OPB = RK * ROWB;                  // bytes per operand chunk (16 KB)
   static_assert(4 * OPB == SMEM_BYTES, "two chunks of two operands");
@@ -90,7 +95,9 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
     off = g.offsets[e];
     cnt = s_cnt[e];
   }
-  const int wm = wave & 1, wn = wave >> 1;  // the wave's 128 (m) x 64 (n) part of the tile
+  const int wm = wave & 1, wn = (wave >> 1) & 3;  // a consumer's 128 (m) x 64 (n) part of the tile
+  const bool producer = wave >= CONSUMERS;
+  const int ptid = tid - CONSUMERS * 64;  // a producer lane's index among the PLANES
   const int lr = lane & 31, lk = lane >> 5;
 
   f32x16 acc[2][4];  // [tn][tm]
@@ -104,8 +111,9 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
   // Loads are unconditional; what lies past the expert's rows or the matrix's columns is read from
   // 16 zero bytes instead (the address is selected, not the data: any instruction on the loaded
   // registers other than the LDS store gets scheduled early and waits for the load there).
-  // Two sets of registers, so that two chunks are on their way from memory at any time (one chunk's
-  // loads take about as long as its MFMAs do: with a single set every chunk waited for its loads).
+  // Two sets of registers in the producers, so that two chunks are on their way from memory at any
+  // time (one chunk's loads take about as long as its MFMAs do: with a single set every chunk waited
+  // for its loads).
   u32x4 ra[2][PER_THREAD], rb[2][PER_THREAD];
   const T* zero_src = reinterpret_cast<const T*>(kZero16);
   auto load_chunk = [&](auto set_c, int r0) {
@@ -113,7 +121,7 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
     int rr[PER_THREAD], arow[PER_THREAD];
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
-      const int r = r0 + (tid + WAVES * 64 * i) / ROW_CHUNKS;
+      const int r = r0 + (ptid + PLANES * i) / ROW_CHUNKS;
       rr[i] = off + (r < cnt ? r : cnt - 1);  // cnt > 0 here
       arow[i] = rr[i];
     }
@@ -123,7 +131,7 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
     }
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
-      const int c = tid + WAVES * 64 * i;
+      const int c = ptid + PLANES * i;
       const int k = c / ROW_CHUNKS, ch = c % ROW_CHUNKS;
       const bool row_ok = r0 + k < cnt;
       const bool a_ok = row_ok && m0 + ch * VEC < M, b_ok = row_ok && n0 + ch * VEC < N;
@@ -139,7 +147,7 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
     uint8_t* sB = sA + OPB;
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
-      const int c = tid + WAVES * 64 * i;
+      const int c = ptid + PLANES * i;
       const int k = c / ROW_CHUNKS, ch = c % ROW_CHUNKS;
       // bf16: chunk ch of row k sits in slot ch ^ ((k & 3) << 2), so that the four consecutive rows
       // a transposing read touches lie 64 bytes apart
@@ -218,25 +226,32 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
   // Every load and store of the loop is unconditional (chunks past the last one load clamped rows
   // and store zeros into the buffer nobody reads any more): behind a condition the compiler cannot
   // count the loads in flight, and waits for all of them, the other set's included, before a store.
-  if (chunks > 0) {
-    load_chunk(Set0{}, 0);
-    load_chunk(Set1{}, RK);
-    store_chunk(Set0{}, 0);
-    load_chunk(Set0{}, 2 * RK);
+  if (producer) {
+    if (chunks > 0) {
+      load_chunk(Set0{}, 0);
+      load_chunk(Set1{}, RK);
+      store_chunk(Set0{}, 0);
+      load_chunk(Set0{}, 2 * RK);
+      lds_barrier();
+    }
+    auto step = [&](int i, auto next_set) {
+      store_chunk(next_set, (i + 1) & 1);
+      load_chunk(next_set, (i + 3) * RK);
+      lds_barrier();  // the loads of the next chunks stay in flight
+    };
+    int ci = 0;
+    for (; ci + 1 < chunks; ci += 2) {
+      step(ci, Set1{});
+      step(ci + 1, Set0{});
+    }
+    if (ci < chunks) step(ci, Set1{});
+    return;  // the consumers write the tile
+  }
+  if (chunks > 0) lds_barrier();
+  for (int i = 0; i < chunks; ++i) {
+    compute_chunk(i & 1);
     lds_barrier();
   }
-  auto step = [&](int i, auto next_set) {
-    store_chunk(next_set, (i + 1) & 1);
-    load_chunk(next_set, (i + 3) * RK);
-    compute_chunk(i & 1);
-    lds_barrier();  // the loads of the next chunks stay in flight
-  };
-  int ci = 0;
-  for (; ci + 1 < chunks; ci += 2) {
-    step(ci, Set1{});
-    step(ci + 1, Set0{});
-  }
-  if (ci < chunks) step(ci, Set1{});
 
   // Accumulator layout: the lane holds row m = lr of fragment tm and columns 8 q + 4 lk + {0..3} of
   // fragment tn in registers 4 q .. 4 q + 3.
