@@ -78,9 +78,12 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
     off = slot * seg_rows;
     cnt = g.dense_rows - off < seg_rows ? g.dense_rows - off : seg_rows;
   } else {
-    __shared__ int s_expert, s_cnt[FS2MOE_MAX_EXPERTS];
+    __shared__ int s_expert, s_cnt[FS2MOE_MAX_EXPERTS], s_off[FS2MOE_MAX_EXPERTS];
     const int mine = tid < g.E ? g.counts[tid] : 0;
-    if (tid < g.E) s_cnt[tid] = mine;
+    if (tid < g.E) {
+      s_cnt[tid] = mine;
+      s_off[tid] = g.offsets[tid];  // with the counts: not a second round trip once the expert is known
+    }
     __syncthreads();
     if (tid < g.E) {
       int rank = 0;
@@ -92,7 +95,7 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
     }
     __syncthreads();
     e = s_expert;
-    off = g.offsets[e];
+    off = s_off[e];
     cnt = s_cnt[e];
   }
   const int wm = wave & 1, wn = (wave >> 1) & 3;  // a consumer's 128 (m) x 64 (n) part of the tile
