@@ -157,8 +157,8 @@ def test_other_expert_activation(gpu_device, dtype, shared):
 
 def test_gradient_and_device_contract(gpu_device):
     # With parameters that require a gradient the call goes through the differentiable function (its
-    # gradients are checked in tests/test_gpu_backward.py) and returns the same values; the stand-alone
-    # expert modules are forward-only and say so.
+    # gradients are checked in tests/test_gpu_backward.py) and returns the same values; so do the expert
+    # modules called by themselves; the row-level entry of the experts is inference only and says so.
     wl = W.make_workload_from_spec(W.small_spec(tokens=8, dtype="bf16"))
     m = build_module(wl, gpu_device)
     x = wl.x.to(torch.bfloat16).to(gpu_device)
@@ -169,8 +169,14 @@ def test_gradient_and_device_contract(gpu_device):
     assert got.requires_grad and torch.equal(got.detach(), want)
     with torch.no_grad():
         assert not m(x).requires_grad
+    xe = x.reshape(1, -1, x.shape[-1]).expand(8, -1, -1).contiguous()
+    with torch.no_grad():
+        want_e = m.experts(xe)
+    got_e = m.experts(xe)
+    assert got_e.requires_grad and torch.equal(got_e.detach(), want_e)
+    counts, offsets = m.experts._uniform_groups(xe.shape[1], xe.device)
     with pytest.raises(RuntimeError, match="forward-only"):
-        m.experts(x.reshape(1, -1, x.shape[-1]).expand(8, -1, -1).contiguous())
+        m.experts.forward_rows(xe.reshape(-1, xe.shape[-1]), counts, offsets)
     with pytest.raises(RuntimeError, match="GPU only"):
         m.requires_grad_(False)(x.cpu())
 
