@@ -44,7 +44,7 @@ template <typename T, bool MAPPED>
 __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
     const T* __restrict__ A, const int32_t* __restrict__ a_map, int lda, const T* __restrict__ B,
     int ldb, T* __restrict__ C, int M, int N, Groups g, int m_tiles, int n_tiles, int seg_rows,
-    float* __restrict__ partial) {
+    float* __restrict__ partial, int paired) {
   using namespace wgk;
   constexpr bool BF16 = sizeof(T) == 2;
   constexpr int RK = BF16 ? 32 : 16;              // rows per chunk
@@ -63,9 +63,33 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
   // XCD b % 8, each with its own L2), so with 8 row blocks the tiles of a slot that share an XCD
   // share their block of A's columns.
   const int per_e = m_tiles * n_tiles;
-  const int slot = blockIdx.x / per_e;
-  const int rem = blockIdx.x - slot * per_e;
-  const int nt = rem / m_tiles, mt = rem - nt * m_tiles;
+  int slot, mt, nt;
+  if (paired) {
+    // Two slots share 2 per_e consecutive blocks, i.e. (per_e being a multiple of 4) whole rounds
+    // of the 8 XCDs: four XCDs per slot, each taking a quarter of the row blocks (or of the column
+    // blocks) with all blocks of the other kind, so that a slot's operand slabs are fetched by 4
+    // L2s with 5 slabs each instead of by 8 with 4 each.  Which half of the XCDs takes the pair's
+    // larger slot alternates from pair to pair.
+    const int pair = blockIdx.x / (2 * per_e);
+    const int i = blockIdx.x - pair * 2 * per_e;
+    const int xcd = i & 7, j = i >> 3, x4 = xcd & 3;
+    slot = 2 * pair + (((xcd >> 2) ^ pair) & 1);
+    if (m_tiles % 4 == 0) {
+      const int q = m_tiles / 4;
+      mt = x4 * q + j % q;
+      nt = j / q;
+    } else {
+      const int q = n_tiles / 4;
+      nt = x4 * q + j % q;
+      mt = j / q;
+    }
+    if (slot >= g.E) return;  // the partner of the last of an odd number of slots
+  } else {
+    slot = blockIdx.x / per_e;
+    const int rem = blockIdx.x - slot * per_e;
+    nt = rem / m_tiles;
+    mt = rem - nt * m_tiles;
+  }
   const int m0 = mt * TM, n0 = nt * TN;
   const bool dense = g.counts == nullptr;
   // Grouped: the experts are taken in descending order of their row counts (ties: lower index
@@ -713,7 +737,11 @@ extern "C" int fs2moe_grouped_wgrad(const void* a, const int32_t* a_row_map, con
   const int slots = counts != nullptr ? E : segments;
   const int seg_rows = (int)(((max_rows + segments - 1) / segments + 15) / 16 * 16);
   float* partial = segments > 1 ? static_cast<float*>(workspace) : nullptr;
-  const int64_t blocks = (int64_t)slots * m_tiles * n_tiles;
+  // grouped, the tile grid divides over four XCDs, and there are enough experts for the two halves
+  // of the XCDs to get the same work over all pairs (with 8 skewed experts they did not: Mixtral's
+  // gradients took 9 % longer): slots in pairs (see the kernel)
+  const int paired = counts != nullptr && E >= 32 && (m_tiles % 4 == 0 || n_tiles % 4 == 0) ? 1 : 0;
+  const int64_t blocks = (int64_t)(paired ? (slots + 1) / 2 * 2 : slots) * m_tiles * n_tiles;
   FS2_REQUIRE(blocks <= 0x7fffffffll, "grouped_wgrad: too many tiles");
   Groups g{counts, offsets, E, (int)max_rows};
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -740,11 +768,11 @@ extern "C" int fs2moe_grouped_wgrad(const void* a, const int32_t* a_row_map, con
     hipLaunchKernelGGL(kb, dim3((unsigned)blocks), dim3(wgk::WAVES * 64), wgk::SMEM_BYTES, st,
                        static_cast<const uint16_t*>(a), a_row_map, M,
                        static_cast<const uint16_t*>(b), N, static_cast<uint16_t*>(dw), M, N, g,
-                       m_tiles, n_tiles, seg_rows, partial);
+                       m_tiles, n_tiles, seg_rows, partial, paired);
   else
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(wgk::WAVES * 64), wgk::SMEM_BYTES, st,
                        static_cast<const float*>(a), a_row_map, M, static_cast<const float*>(b), N,
-                       static_cast<float*>(dw), M, N, g, m_tiles, n_tiles, seg_rows, partial);
+                       static_cast<float*>(dw), M, N, g, m_tiles, n_tiles, seg_rows, partial, paired);
   if (int rc = check_launch("grouped_wgrad")) return rc;
   if (segments > 1) {
     const int64_t n = (int64_t)M * N;
