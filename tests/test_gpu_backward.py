@@ -301,7 +301,13 @@ def test_backward_twice_gives_the_same_gradients(gpu_device):
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
-@pytest.mark.parametrize("rows,m,n", [([5, 0, 300, 64, 1], 64, 96), ([130, 257], 136, 264), ([33], 8, 8), ([0, 0], 128, 128)])
+@pytest.mark.parametrize("rows,m,n", [
+    ([5, 0, 300, 64, 1], 64, 96), ([130, 257], 136, 264), ([33], 8, 8), ([0, 0], 128, 128),
+    # 32 experts or more: two experts share a round of blocks when the tile grid divides by four
+    # (1024 / 256 row blocks here, then 4 column blocks); an odd count leaves the last one alone
+    ([(7 * i) % 90 for i in range(33)], 1024, 264), ([(11 * i) % 70 for i in range(35)], 72, 1024),
+    ([40 + i for i in range(32)], 520, 520),
+])
 def test_grouped_wgrad_matches_torch(gpu_device, dtype, rows, m, n):
     _say("grouped_wgrad", dtype, rows, m, n)
     dt = TORCH_DTYPE[dtype]
