@@ -15,7 +15,7 @@ from torch import Tensor
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfs2moe.so")
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
@@ -53,6 +53,12 @@ _PROTOTYPES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
          c_void_p, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p,
          c_void_p],
+    ),
+    "fs2moe_grouped_swiglu_rows": (
+        c_int32,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p,
+         c_int32, c_void_p],
     ),
     "fs2moe_grouped_swiglu_fuses_gather": (c_int32, [c_int32, c_int32, c_int32, c_int32]),
     "fs2moe_grouped_swiglu_keeps": (c_int32, [c_int32, c_int32, c_int64, c_int32]),
@@ -393,8 +399,13 @@ def grouped_swiglu(
     num_experts: int,
     scales: tuple[Tensor, Tensor, Tensor] | None = None,
     row_map: Tensor | None = None,
+    rows_per_expert: int = 0,
 ) -> tuple[Tensor, Tensor]:
     """Returns ``(ye, h)`` for the rows of ``xe`` (rows, D).
+
+    ``rows_per_expert``: an upper bound on the rows of any one expert when the caller knows one
+    (the number of tokens is one), else 0; with 1..4 and bf16 weights the products run as streams
+    over the weights instead of as GEMM tiles (``fs2moe_grouped_swiglu_rows``).
 
     With ``row_map`` (int32, one entry per row: ``Dispatched.perm``) ``xe`` is the token matrix
     ``(T, D)`` and row ``r`` of the experts' input is ``xe[row_map[r]]``: the gather is fused into
@@ -435,12 +446,12 @@ def grouped_swiglu(
     h = torch.empty((rows, f), dtype=xe.dtype, device=xe.device)
     ye = torch.empty((rows, d), dtype=xe.dtype, device=xe.device)
     sg, su, sd = scales if scales is not None else (None, None, None)
-    rc = lib.fs2moe_grouped_swiglu(
+    rc = lib.fs2moe_grouped_swiglu_rows(
         _ptr(xe), _ptr(row_map), _ptr(counts), _ptr(offsets), _ptr(w_gate), _ptr(w_up),
         _ptr(w_down), _ptr(sg), _ptr(su), _ptr(sd), num_experts, d, f, rows, dtype_code(xe.dtype),
-        dtype_code(w_gate.dtype), _ptr(h), _ptr(ye), _stream(),
+        dtype_code(w_gate.dtype), _ptr(h), _ptr(ye), int(rows_per_expert), _stream(),
     )
-    _check(rc, "fs2moe_grouped_swiglu")
+    _check(rc, "fs2moe_grouped_swiglu_rows")
     return ye, h
 
 

@@ -22,6 +22,7 @@
 #include "tile_map.h"
 #include "experts_dma.h"
 #include "experts_fp8.h"
+#include "experts_gemv.h"
 
 namespace fs2moe {
 
@@ -396,11 +397,67 @@ static bool dma_offsets_fit(int64_t rows_bound, int D, int F) {
   return rows_bound * wide * 2 <= 0xffffffffll && (int64_t)D * F * 2 <= 0xffffffffll;
 }
 
+// The streaming pair for at most `rows_hint` rows per expert: see experts_gemv.h.  Measured on the
+// Qwen3 layer shape (bf16 weights, whole layer, against the GEMM tiles): 1 token 44-47 against 69 us,
+// 2 tokens 52 against 70, 3 tokens 56 against 71, 4 tokens 61 against 72; from 5 rows on the vector
+// ALUs fall behind (8 tokens: 95 against 84 us), so the bound stops at 4.
+#ifndef FS2MOE_GEMV_MAX_ROWS
+#define FS2MOE_GEMV_MAX_ROWS 4
+#endif
+static bool gemv_applies(int act_dtype, int D, int F, const Groups& g, int rows_hint) {
+  if (act_dtype != FS2MOE_BF16 || g.counts == nullptr || rows_hint < 1 ||
+      rows_hint > FS2MOE_GEMV_MAX_ROWS)
+    return false;
+  const int r = rows_hint <= 1 ? 1 : rows_hint <= 2 ? 2 : 4;
+  return gemv::fits(D > F ? D : F, r);
+}
+
+template <int R>
+static int launch_gemv_pair_r(const void* x, const int32_t* row_map, const Groups& g,
+                              const void* w_gate, const void* w_up, const void* w_down, int D, int F,
+                              void* h, void* y, hipStream_t stream) {
+  using namespace gemv;
+  auto k1 = glu_gemv_bf16_kernel<true, R>;
+  auto k2 = glu_gemv_bf16_kernel<false, R>;
+  static bool attr_set = false;  // benign race: setting the attribute is idempotent
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(k1),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS_BYTES) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(k2),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS_BYTES) != hipSuccess) {
+      set_error("experts: cannot reserve %d bytes of LDS", MAX_LDS_BYTES);
+      return FS2MOE_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  const uint16_t* xp = static_cast<const uint16_t*>(x);
+  hipLaunchKernelGGL(k1, dim3((unsigned)((F + COLS - 1) / COLS), (unsigned)g.E), dim3(threads(R)),
+                     (size_t)R * D * 2, stream, xp, row_map, D, static_cast<const uint16_t*>(w_gate),
+                     static_cast<const uint16_t*>(w_up), static_cast<uint16_t*>(h), F, D, F,
+                     g.counts, g.offsets);
+  if (int rc = check_launch("glu_gemv_bf16<gate,up>")) return rc;
+  hipLaunchKernelGGL(k2, dim3((unsigned)((D + COLS - 1) / COLS), (unsigned)g.E), dim3(threads(R)),
+                     (size_t)R * F * 2, stream, static_cast<const uint16_t*>(h),
+                     static_cast<const int32_t*>(nullptr), F, static_cast<const uint16_t*>(w_down),
+                     static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(y), D, F, D,
+                     g.counts, g.offsets);
+  return check_launch("glu_gemv_bf16<down>");
+}
+
+// rows_hint: an upper bound on the rows of any one expert when the caller knows one (the number of
+// tokens is one: a token takes an expert at most once), else 0.
 template <int BLAYOUT>
 static int launch_glu(const void* x, const int32_t* row_map, const Groups& g, int64_t rows_bound,
                       const void* w_gate, const void* w_up, const void* w_down, int D, int F,
-                      int act_dtype, void* h, void* y, hipStream_t stream) {
+                      int act_dtype, void* h, void* y, hipStream_t stream, int rows_hint = 0) {
   const int groups = g.counts ? g.E : 0;
+  if constexpr (BLAYOUT == FS2MOE_W_IN_OUT) {
+    if (gemv_applies(act_dtype, D, F, g, rows_hint)) {
+      if (rows_hint <= 1) return launch_gemv_pair_r<1>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
+      if (rows_hint <= 2) return launch_gemv_pair_r<2>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
+      return launch_gemv_pair_r<4>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
+    }
+  }
   if (dma_path_applies(act_dtype, D, F) && dma_offsets_fit(rows_bound, D, F))
     return launch_dma_pair<BLAYOUT>(x, row_map, g, rows_bound, w_gate, w_up, w_down, nullptr, nullptr,
                                     nullptr, D, F, h, y, stream);
@@ -491,14 +548,15 @@ extern "C" int fs2moe_grouped_swiglu_keep(const void* xe, const int32_t* row_map
                                           static_cast<hipStream_t>(stream), g, u);
 }
 
-extern "C" int fs2moe_grouped_swiglu(const void* xe, const int32_t* row_map, const int32_t* counts,
-                                     const int32_t* offsets, const void* w_gate, const void* w_up,
-                                     const void* w_down, const float* s_gate, const float* s_up,
-                                     const float* s_down, int32_t E, int32_t D, int32_t F,
-                                     int64_t max_rows, int32_t act_dtype, int32_t w_dtype, void* h,
-                                     void* ye, void* stream) {
+static int grouped_swiglu_impl(const void* xe, const int32_t* row_map, const int32_t* counts,
+                               const int32_t* offsets, const void* w_gate, const void* w_up,
+                               const void* w_down, const float* s_gate, const float* s_up,
+                               const float* s_down, int32_t E, int32_t D, int32_t F,
+                               int64_t max_rows, int32_t act_dtype, int32_t w_dtype, void* h,
+                               void* ye, int32_t rows_hint, void* stream) {
   FS2_REQUIRE(xe && counts && offsets && w_gate && w_up && w_down && h && ye,
               "grouped_swiglu: null pointer");
+  FS2_REQUIRE(rows_hint >= 0, "grouped_swiglu: rows_per_expert=%d", rows_hint);
   FS2_REQUIRE(E >= 1 && E <= FS2MOE_MAX_EXPERTS, "grouped_swiglu: E=%d outside [1, %d]", E,
               FS2MOE_MAX_EXPERTS);
   FS2_REQUIRE(D > 0 && F > 0 && D % 8 == 0 && F % 8 == 0,
@@ -585,7 +643,28 @@ extern "C" int fs2moe_grouped_swiglu(const void* xe, const int32_t* row_map, con
   if (max_rows == 0) return FS2MOE_OK;
   Groups g{counts, offsets, E, 0};
   return launch_glu<FS2MOE_W_IN_OUT>(xe, row_map, g, max_rows, w_gate, w_up, w_down, D, F, act_dtype,
-                                     h, ye, static_cast<hipStream_t>(stream));
+                                     h, ye, static_cast<hipStream_t>(stream), rows_hint);
+}
+
+extern "C" int fs2moe_grouped_swiglu(const void* xe, const int32_t* row_map, const int32_t* counts,
+                                     const int32_t* offsets, const void* w_gate, const void* w_up,
+                                     const void* w_down, const float* s_gate, const float* s_up,
+                                     const float* s_down, int32_t E, int32_t D, int32_t F,
+                                     int64_t max_rows, int32_t act_dtype, int32_t w_dtype, void* h,
+                                     void* ye, void* stream) {
+  return grouped_swiglu_impl(xe, row_map, counts, offsets, w_gate, w_up, w_down, s_gate, s_up, s_down,
+                             E, D, F, max_rows, act_dtype, w_dtype, h, ye, 0, stream);
+}
+
+extern "C" int fs2moe_grouped_swiglu_rows(const void* xe, const int32_t* row_map,
+                                          const int32_t* counts, const int32_t* offsets,
+                                          const void* w_gate, const void* w_up, const void* w_down,
+                                          const float* s_gate, const float* s_up,
+                                          const float* s_down, int32_t E, int32_t D, int32_t F,
+                                          int64_t max_rows, int32_t act_dtype, int32_t w_dtype,
+                                          void* h, void* ye, int32_t rows_per_expert, void* stream) {
+  return grouped_swiglu_impl(xe, row_map, counts, offsets, w_gate, w_up, w_down, s_gate, s_up, s_down,
+                             E, D, F, max_rows, act_dtype, w_dtype, h, ye, rows_per_expert, stream);
 }
 
 // One grouped (or dense) GEMM, C = A @ B_e, on the kernels of the SwiGLU pair's second half.

@@ -201,11 +201,14 @@ class GroupedExpertNetwork(ExpertNetwork):
         return _abi.fuses_gather(self.model_dim, self.inner_dim, act_dtype, self.gate_proj.dtype)
 
     def forward_rows(
-        self, xe: Tensor, counts: Tensor, offsets: Tensor, row_map: Tensor | None = None
+        self, xe: Tensor, counts: Tensor, offsets: Tensor, row_map: Tensor | None = None,
+        rows_per_expert: int = 0,
     ) -> Tensor:
         """Runs every expert on its block of rows of ``xe`` (rows, D); with ``row_map``, row ``r``
-        is ``xe[row_map[r]]`` and ``xe`` is the token matrix.  Inference only (the training
-        paths are :meth:`forward` and the layer's)."""
+        is ``xe[row_map[r]]`` and ``xe`` is the token matrix.  ``rows_per_expert``: an upper bound
+        on any expert's rows when the caller knows one (the number of tokens is one), else 0; up to 8
+        the bf16 experts run as streams over their weights.  Inference only (the training paths are
+        :meth:`forward` and the layer's)."""
         _require_forward_only(xe, self.gate_proj, self.inner_proj, self.output_proj)
         if not self.has_fused_gate:
             # experts.py:107-112 with the module's own activation between the library's GEMMs
@@ -227,6 +230,7 @@ class GroupedExpertNetwork(ExpertNetwork):
         ye, _ = _abi.grouped_swiglu(
             xe, counts, offsets, self.gate_proj.detach(), self.inner_proj.detach(),
             self.output_proj.detach(), self.num_local_experts, row_map=row_map,
+            rows_per_expert=rows_per_expert,
         )
         return ye
 
@@ -615,10 +619,13 @@ class MoE(FeedForwardNetwork):
         disp = _abi.dispatch(
             idx, w, x, ex.num_local_experts, self.tile_m, scale_input, gather=not fused
         )
+        # a token takes an expert at most once: with up to 8 tokens no expert has more rows than that
+        # (what the whole-layer call passes on as well)
+        hint = dict(rows_per_expert=x.shape[0]) if isinstance(ex, GroupedExpertNetwork) and x.shape[0] <= 8 else {}
         if fused:
-            ye = ex.forward_rows(x, disp.counts, disp.offsets, row_map=disp.perm)
+            ye = ex.forward_rows(x, disp.counts, disp.offsets, row_map=disp.perm, **hint)
         else:
-            ye = ex.forward_rows(disp.xe, disp.counts, disp.offsets)
+            ye = ex.forward_rows(disp.xe, disp.counts, disp.offsets, **hint)
         base = None
         if self.shared_expert is not None:
             base = self.shared_expert(x)

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FS2MOE_ABI_VERSION 11
+#define FS2MOE_ABI_VERSION 12
 
 /* element types */
 #define FS2MOE_F32 0
@@ -157,6 +157,23 @@ int fs2moe_grouped_swiglu(const void* xe, const int32_t* row_map, const int32_t*
                           const void* w_down, const float* s_gate, const float* s_up,
                           const float* s_down, int32_t E, int32_t D, int32_t F, int64_t max_rows,
                           int32_t act_dtype, int32_t w_dtype, void* h, void* ye, void* stream);
+
+/*
+ * fs2moe_grouped_swiglu for a caller that knows an upper bound on the rows of any one expert
+ * (rows_per_expert; 0: no bound known, then this is fs2moe_grouped_swiglu).  The number of tokens is
+ * such a bound (torch.topk of moe.py:113 gives a token an expert at most once), which is what a
+ * decode step of a few sequences (generation/: one token per sequence and step) has to offer: with
+ * a bound of 1..4 and bf16 weights the two products run as streams over the active experts' weights
+ * on the vector ALUs (no LDS tiles, no matrix pipe) instead of as GEMM tiles (larger bounds: as 0).  Same arguments and
+ * results (to the order of f32 additions) otherwise; a count above the bound is still computed
+ * correctly, only slowly.
+ */
+int fs2moe_grouped_swiglu_rows(const void* xe, const int32_t* row_map, const int32_t* counts,
+                               const int32_t* offsets, const void* w_gate, const void* w_up,
+                               const void* w_down, const float* s_gate, const float* s_up,
+                               const float* s_down, int32_t E, int32_t D, int32_t F,
+                               int64_t max_rows, int32_t act_dtype, int32_t w_dtype, void* h,
+                               void* ye, int32_t rows_per_expert, void* stream);
 
 /* 1 if fs2moe_grouped_swiglu accepts a row_map for these sizes and types, else 0. */
 int fs2moe_grouped_swiglu_fuses_gather(int32_t D, int32_t F, int32_t act_dtype, int32_t w_dtype);

@@ -278,6 +278,61 @@ def test_grouped_swiglu_matches_oracle(gpu_device, dtype, rows_per_expert, d, f)
         assert_output_close(ye[lo : lo + n], y_full, dtype, f"expert {ex}")
 
 
+@pytest.mark.parametrize(
+    "bound,rows_per_expert,d,f",
+    [
+        (1, [1, 0, 1, 1, 0, 0, 1, 1], 2048, 768),   # one decoding sequence at the Qwen3 shape
+        (1, [1, 1], 72, 40),                          # K not a multiple of the 128 rows a step takes
+        (2, [2, 0, 1, 2], 256, 136),
+        (4, [3, 4, 0, 1, 4, 2], 128, 200),
+        (8, [8, 5, 0, 7, 1, 8, 3], 320, 192),
+        (8, [(3 * i) % 9 for i in range(128)], 64, 64),
+        (4, [9, 4, 13, 0, 1], 128, 64),               # counts above the bound: walked again, still right
+        (4, [4, 2], 8192, 64),                        # the longest K whose four rows fit LDS
+    ],
+)
+def test_grouped_swiglu_with_a_bound_on_the_rows_per_expert(gpu_device, bound, rows_per_expert, d, f):
+    """``fs2moe_grouped_swiglu_rows``: with a bound of 1..4 rows per expert and bf16 weights the two
+    products stream the weights through the vector ALUs (larger bounds take the GEMM kernels).  Each
+    expert against the oracle's SwiGLU in f64; rows read through a map give the same bits."""
+    _say("grouped_swiglu_rows", bound, rows_per_expert[:8], d, f)
+    counts, offsets, xe, wg, wu, wd = _expert_case("bf16", rows_per_expert, d, f, seed=bound + d + f)
+    e = len(rows_per_expert)
+    dev = gpu_device
+    bf = torch.bfloat16
+    args = (counts.to(dev), offsets.to(dev), wg.to(bf).to(dev), wu.to(bf).to(dev), wd.to(bf).to(dev), e)
+    ye, h = _abi.grouped_swiglu(xe.to(bf).to(dev), *args, rows_per_expert=bound)
+    for ex in range(e):
+        lo, n = int(offsets[ex]), int(counts[ex])
+        if n == 0:
+            continue
+        u = xe[lo : lo + n].double()
+        h_ref = torch.nn.functional.silu(u @ wg[ex * d : (ex + 1) * d].double()) * (u @ wu[ex * d : (ex + 1) * d].double())
+        assert_output_close(h[lo : lo + n], h_ref, "bf16", f"h of expert {ex}")
+        y_ref = h[lo : lo + n].double().cpu() @ wd[ex * f : (ex + 1) * f].double()
+        assert_output_close(ye[lo : lo + n], y_ref, "bf16", f"ye of expert {ex}")
+        y_full = O.glu_expert(u, wg[ex * d : (ex + 1) * d].double(), wu[ex * d : (ex + 1) * d].double(), wd[ex * f : (ex + 1) * f].double())
+        assert_output_close(ye[lo : lo + n], y_full, "bf16", f"expert {ex}")
+    # through a row map: rows scattered over a larger matrix, same bits
+    total = xe.shape[0]
+    g = torch.Generator().manual_seed(5)
+    src_rows = torch.randperm(total + 11, generator=g)[:total]
+    src = torch.randn(total + 11, d, generator=g).to(bf)
+    src[src_rows] = xe.to(bf)
+    ye2, h2 = _abi.grouped_swiglu(src.to(dev), *args, row_map=src_rows.to(torch.int32).to(dev), rows_per_expert=bound)
+    for ex in range(e):
+        lo, n = int(offsets[ex]), int(counts[ex])
+        assert torch.equal(ye2[lo : lo + n], ye[lo : lo + n]) and torch.equal(h2[lo : lo + n], h[lo : lo + n])
+    # bounds outside 1..4 take the other kernels; a negative bound is refused
+    ye3, _ = _abi.grouped_swiglu(xe.to(bf).to(dev), *args, rows_per_expert=9)
+    ye4, _ = _abi.grouped_swiglu(xe.to(bf).to(dev), *args)
+    for ex in range(e):
+        lo, n = int(offsets[ex]), int(counts[ex])
+        assert torch.equal(ye3[lo : lo + n], ye4[lo : lo + n])
+    with pytest.raises(_abi.Fs2MoeError, match="rows_per_expert"):
+        _abi.grouped_swiglu(xe.to(bf).to(dev), *args, rows_per_expert=-1)
+
+
 def test_grouped_swiglu_row_map_equals_gathered_rows(gpu_device):
     """Reading the rows through dispatch's permutation gives bit for bit what the gathered copy gives."""
     _say("grouped_swiglu row_map")
