@@ -124,13 +124,23 @@ class GroupedExpertNetwork(ExpertNetwork):
         for name in self._FP8_NAMES:
             if hasattr(self, f"_{name}_bits"):
                 delattr(self, f"_{name}_bits")
+        self.__dict__.pop("_fp8_view_cache", None)
 
     def _fp8_view(self, name: str) -> Tensor:
         bits = getattr(self, f"_{name}_bits")
+        # the typed view is kept for as long as the buffer object stays the same (a view costs a few
+        # microseconds of host time, and a decode step takes six of them per layer); Module.to(),
+        # load_fp8_weights and clear_fp8_weights all install new buffer objects
+        cache = self.__dict__.setdefault("_fp8_view_cache", {})
+        hit = cache.get(name)
+        if hit is not None and hit[0] is bits:
+            return hit[1]
         want = torch.uint8 if name.endswith("_q") else torch.int32
         if bits.dtype != want:
             raise RuntimeError(f"the fp8 buffer {name} was cast to {bits.dtype}; quantise again")
-        return bits.view(torch.float8_e4m3fn if name.endswith("_q") else torch.float32)
+        view = bits.view(torch.float8_e4m3fn if name.endswith("_q") else torch.float32)
+        cache[name] = (bits, view)
+        return view
 
     gate_q = property(lambda self: self._fp8_view("gate_q"))
     inner_q = property(lambda self: self._fp8_view("inner_q"))
@@ -646,7 +656,7 @@ class MoE(FeedForwardNetwork):
         if self.tp_gang is not None:
             raise NotImplementedError("tensor-parallel reduction is not part of the single-GPU path")
         _require_device(seqs)
-        if not allow_grad:
+        if not allow_grad and torch.is_grad_enabled():  # (walking the parameters costs host time)
             _require_forward_only(seqs, *self.parameters())
         if seqs.dtype != self.router.dtype:
             hint = ""
