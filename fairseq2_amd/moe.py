@@ -131,15 +131,21 @@ class GroupedExpertNetwork(ExpertNetwork):
         # the typed view is kept for as long as the buffer object stays the same (a view costs a few
         # microseconds of host time, and a decode step takes six of them per layer); Module.to(),
         # load_fp8_weights and clear_fp8_weights all install new buffer objects
-        cache = self.__dict__.setdefault("_fp8_view_cache", {})
-        hit = cache.get(name)
-        if hit is not None and hit[0] is bits:
-            return hit[1]
+        # (not while a compiler traces the call: the view is then part of the trace)
+        tracing = torch.compiler.is_compiling()
+        if not tracing:
+            cache = self.__dict__.get("_fp8_view_cache")
+            if cache is None:
+                cache = self.__dict__["_fp8_view_cache"] = {}
+            hit = cache.get(name)
+            if hit is not None and hit[0] is bits:
+                return hit[1]
         want = torch.uint8 if name.endswith("_q") else torch.int32
         if bits.dtype != want:
             raise RuntimeError(f"the fp8 buffer {name} was cast to {bits.dtype}; quantise again")
         view = bits.view(torch.float8_e4m3fn if name.endswith("_q") else torch.float32)
-        cache[name] = (bits, view)
+        if not tracing:
+            cache[name] = (bits, view)
         return view
 
     gate_q = property(lambda self: self._fp8_view("gate_q"))
