@@ -271,9 +271,11 @@ class GroupedExpertNetwork(ExpertNetwork):
 
             ye = GroupedExpertsFunction.apply(
                 x.reshape(e * n, d).contiguous(), counts, offsets, *params, e,
-                None if self.has_fused_gate else self.activation)
+                None if self.has_fused_gate else self.activation, n if n <= 8 else 0)
             return ye.view(e, n, d)
-        return self.forward_rows(x.reshape(e * n, d).contiguous(), counts, offsets).view(e, n, d)
+        # (every expert has exactly n rows: a bound the library can use when it is small)
+        return self.forward_rows(x.reshape(e * n, d).contiguous(), counts, offsets,
+                                 rows_per_expert=n if n <= 8 else 0).view(e, n, d)
 
     def _uniform_groups(self, n: int, device: torch.device) -> tuple[Tensor, Tensor]:
         """counts / offsets of ``n`` rows for every expert, built once per (n, device) so that the

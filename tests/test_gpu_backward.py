@@ -625,7 +625,7 @@ def test_gradients_through_the_normalisation_compose(gpu_device, dtype):
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 @pytest.mark.parametrize("e,n,d,f,act", [(6, 37, 128, 192, None), (4, 300, 256, 128, None), (3, 50, 72, 40, None),
-                                         (4, 64, 128, 64, "gelu")])
+                                         (4, 64, 128, 64, "gelu"), (5, 3, 128, 192, None), (2, 1, 64, 64, None)])
 def test_grouped_expert_network_alone_is_differentiable(gpu_device, dtype, e, n, d, f, act):
     """``GroupedExpertNetwork.forward((E, n, D))`` (``experts.py:201-213``) under autograd: the
     gradients of its input and of the three weights against float64 autograd through the oracle's
