@@ -65,6 +65,12 @@ def test_argument_errors_are_reported_without_touching_the_gpu(lib):
     # experts: dims not multiples of 8
     rc = lib.fs2moe_grouped_swiglu(fake, None, fake, fake, fake, fake, fake, None, None, None, 4, 60, 64, 128, _abi.BF16, _abi.BF16, fake, fake, None)
     assert rc == -1 and b"multiples of 8" in lib.fs2moe_last_error()
+    # the variant with a bound on the rows per expert checks the same things, and the bound
+    rc = lib.fs2moe_grouped_swiglu_rows(fake, None, fake, fake, fake, fake, fake, None, None, None, 4, 60, 64, 128, _abi.BF16, _abi.BF16, fake, fake, 2, None)
+    assert rc == -1 and b"multiples of 8" in lib.fs2moe_last_error()
+    rc = lib.fs2moe_grouped_swiglu_rows(fake, None, fake, fake, fake, fake, fake, None, None, None, 4, 64, 64, 128, _abi.BF16, _abi.BF16, fake, fake, -1, None)
+    assert rc == -1 and b"rows_per_expert" in lib.fs2moe_last_error()
+    assert lib.fs2moe_grouped_swiglu_rows(fake, None, fake, fake, fake, fake, fake, None, None, None, 4, 64, 64, 0, _abi.BF16, _abi.BF16, fake, fake, 2, None) == 0
     # the fused gather exists for bf16 activations with D and F multiples of 64 (bf16 or e4m3
     # weights), and nowhere else
     assert lib.fs2moe_grouped_swiglu_fuses_gather(2048, 768, _abi.BF16, _abi.BF16) == 1
