@@ -277,12 +277,14 @@ def test_module_fp8_quantiser_matches_the_workload_quantiser(gpu_device):
         assert float((qa.float() - qb.float()).abs().max()) <= 32.0  # at most one e4m3 step (top binade)
 
 
-def test_graphed_forward_replays_match_eager(gpu_device):
+@pytest.mark.parametrize("tokens", [96, 3])
+def test_graphed_forward_replays_match_eager(gpu_device, tokens):
     """A captured graph of the layer, replayed several times with eager work and synchronisations
-    between the replays, gives the eager result bit for bit every time."""
+    between the replays, gives the eager result bit for bit every time (96 tokens: the GEMM kernels;
+    3 tokens: the experts as streams over their weights)."""
     from fairseq2_amd import GraphedForward
 
-    wl = W.make_workload_from_spec(W.small_spec(dtype="bf16", shared=True, seed=11))
+    wl = W.make_workload_from_spec(W.small_spec(dtype="bf16", shared=True, seed=11, tokens=tokens))
     m = build_module(wl, gpu_device)
     xs = [wl.x.to(torch.bfloat16).to(gpu_device)]
     g = torch.Generator().manual_seed(5)
