@@ -134,21 +134,20 @@ int forward_impl(bool normed, const void* x_in, const void* norm_weight, float n
                      (w_dtype == FS2MOE_FP8_E4M3 || widest <= 0xffffffffll);
   const ForwardBuffers b = carve_forward(workspace, T, D, E, K, F, shared ? F_shared : 0, tile_m,
                                          act_dtype, !fused, normed);
-  if (normed) {
-    if (int rc = fs2moe_router_topk_norm(x, norm_weight, norm_eps, b.xn, router, router_bias, T, D,
-                                         E, K, act_dtype, score_fn, renormalize, b.topk_idx,
-                                         b.topk_w, nullptr, b.router_ws, b.router_ws_bytes, stream))
+  // (with a few tokens and no rows to copy the router's kernel dispatches as well)
+  fs2moe::DispatchAfterRouter disp = {tile_m, b.max_rows, b.counts, b.offsets, b.perm, b.inv_perm, false};
+  if (int rc = fs2moe::router_then_dispatch(x, normed ? norm_weight : nullptr, normed ? norm_eps : 0.f,
+                                    normed ? b.xn : nullptr, router, router_bias, T, D, E, K,
+                                    act_dtype, score_fn, renormalize, b.topk_idx, b.topk_w,
+                                    b.router_ws, b.router_ws_bytes, b.xe == nullptr ? &disp : nullptr,
+                                    stream))
+    return rc;
+  if (normed) x = b.xn;
+  if (!disp.done)
+    if (int rc = fs2moe_dispatch(b.topk_idx, b.topk_w, x, T, K, E, D, tile_m, act_dtype,
+                                 scale_input, b.max_rows, b.counts, b.offsets, b.perm, b.inv_perm,
+                                 b.xe, b.disp_ws, b.disp_ws_bytes, stream))
       return rc;
-    x = b.xn;
-  } else if (int rc = fs2moe_router_topk(x, router, router_bias, T, D, E, K, act_dtype, score_fn,
-                                         renormalize, b.topk_idx, b.topk_w, nullptr, b.router_ws,
-                                         b.router_ws_bytes, stream)) {
-    return rc;
-  }
-  if (int rc = fs2moe_dispatch(b.topk_idx, b.topk_w, x, T, K, E, D, tile_m, act_dtype, scale_input,
-                               b.max_rows, b.counts, b.offsets, b.perm, b.inv_perm, b.xe, b.disp_ws,
-                               b.disp_ws_bytes, stream))
-    return rc;
   // (a token takes an expert at most once: with up to 8 tokens no expert has more rows than that)
   if (int rc = fs2moe_grouped_swiglu_rows(fused ? x : b.xe, fused ? b.perm : nullptr, b.counts,
                                           b.offsets, w_gate, w_up, w_down, s_gate, s_up, s_down, E,

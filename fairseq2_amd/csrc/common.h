@@ -168,6 +168,22 @@ int check_launch(const char* what);
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline int elem_size(int dtype) { return dtype == FS2MOE_F32 ? 4 : dtype == FS2MOE_BF16 ? 2 : 1; }
 
+// Where the whole-layer call wants its dispatch (no rows copied): with at most 32 bf16 tokens the
+// router's finishing kernel ends with it and sets `done`; at any other size the router leaves
+// `done` false and the caller runs fs2moe_dispatch.  Either way the arrays hold the same values.
+struct DispatchAfterRouter {
+  int tile_m;
+  int64_t max_rows;
+  int32_t *counts, *offsets, *perm, *inv_perm;
+  bool done;
+};
+// fs2moe_router_topk (xn null) or fs2moe_router_topk_norm, without the logits output
+int router_then_dispatch(const void* x, const void* norm_w, float norm_eps, void* xn,
+                         const void* router, const float* bias, int32_t T, int32_t D, int32_t E,
+                         int32_t K, int32_t act_dtype, int32_t score_fn, int32_t renormalize,
+                         int32_t* topk_idx, float* topk_w, void* workspace, int64_t workspace_bytes,
+                         DispatchAfterRouter* disp, void* stream);
+
 }  // namespace fs2moe
 
 #define FS2_REQUIRE(cond, ...)          \

@@ -7,11 +7,9 @@
 // bits below its token, and the block's base is a prefix over the per-block counts.  No float or
 // order-dependent atomics are involved; the result is the expert-major, token-ascending order.
 #include "common.h"
+#include "dispatch_small.h"
 
 namespace fs2moe {
-
-constexpr int kDispTok = 256;  // tokens per block in the counting pass (= threads per block)
-constexpr int kDispWords = kDispTok / 32;
 
 // The experts of token t, -1 where there is none (t past T, k past K, an index outside [0, E)).
 // Every load is issued, from an address inside the array, before any result is looked at: a load
@@ -229,75 +227,9 @@ __global__ __launch_bounds__(kDispTok) void dispatch_small_kernel(
     int32_t* __restrict__ counts, int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
     int32_t* __restrict__ inv_perm) {
   extern __shared__ uint32_t s_mem[];
-  uint32_t* s_bits = s_mem;                    // [E][kDispWords] membership bitmaps
-  uint32_t* s_pref = s_mem + E * kDispWords;   // [E][kDispWords] members in the words below
-  int32_t* s_off = reinterpret_cast<int32_t*>(s_pref + E * kDispWords);  // [E + 1]
   __shared__ int32_t s_wave_tot[4];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int i = tid; i < E * kDispWords; i += kDispTok) s_bits[i] = 0u;
-  __syncthreads();
-  const int t = tid;
-  const int word = tid >> 5;
-  const uint32_t bit = 1u << (tid & 31);
-  int ek[FS2MOE_MAX_TOP_K];
-  load_token_experts(topk_idx, t, T, K, E, ek);
-#pragma unroll
-  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k)
-    if (ek[k] >= 0) atomicOr(&s_bits[ek[k] * kDispWords + word], bit);
-  __syncthreads();
-  for (int i = tid; i < E * kDispWords; i += kDispTok) {
-    const int e = i / kDispWords, w = i % kDispWords;
-    uint32_t c = 0;
-    for (int j = 0; j < w; ++j) c += __popc(s_bits[e * kDispWords + j]);
-    s_pref[i] = c;
-  }
-  __syncthreads();
-  // counts and tile-padded offsets: thread e, a block-wide exclusive scan (E <= 256 = block size)
-  int cnt = 0, padded = 0;
-  if (tid < E) {
-    const int i = tid * kDispWords + kDispWords - 1;
-    cnt = (int)(s_pref[i] + __popc(s_bits[i]));
-    counts[tid] = cnt;
-    padded = (cnt + tile_m - 1) / tile_m * tile_m;
-  }
-  int incl = padded;
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    int v = __shfl_up(incl, off, kWave);
-    if (lane >= off) incl += v;
-  }
-  if (lane == 63) s_wave_tot[wave] = incl;
-  __syncthreads();
-  int base = 0;
-  for (int w = 0; w < wave; ++w) base += s_wave_tot[w];
-  if (tid < E) {
-    offsets[tid] = base + incl - padded;
-    s_off[tid] = base + incl - padded;
-  }
-  if (tid == E - 1) {
-    offsets[E] = base + incl;
-    s_off[E] = base + incl;
-  }
-  __syncthreads();
-  // pairs
-#pragma unroll
-  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) {
-    if (k < K && t < T) {
-      const size_t p = (size_t)t * K + k;
-      if (ek[k] < 0) {
-        inv_perm[p] = -1;
-      } else {
-        const int i = ek[k] * kDispWords + word;
-        const int row = s_off[ek[k]] + (int)(s_pref[i] + __popc(s_bits[i] & (bit - 1u)));
-        inv_perm[p] = row;
-        perm[row] = t;
-      }
-    }
-  }
-  // padding rows of expert tid, then the rows beyond offsets[E]
-  if (tid < E)
-    for (int r = s_off[tid] + cnt; r < s_off[tid + 1]; ++r) perm[r] = -1;
-  for (int64_t r = (int64_t)s_off[E] + tid; r < max_rows; r += kDispTok) perm[r] = -1;
+  dispatch_small_block(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm, s_mem,
+                       s_wave_tot, threadIdx.x, kDispTok);
 }
 
 }  // namespace fs2moe
@@ -347,7 +279,7 @@ extern "C" int fs2moe_dispatch(const int32_t* topk_idx, const float* topk_w, con
 
   if (nb == 1 && xe == nullptr) {
     hipLaunchKernelGGL(dispatch_small_kernel, dim3(1), dim3(kDispTok),
-                       ((size_t)E * kDispWords * 2 + E + 1) * sizeof(uint32_t), s, topk_idx, T, K, E,
+                       dispatch_small_lds_words(E) * sizeof(uint32_t), s, topk_idx, T, K, E,
                        tile_m, max_rows, counts, offsets, perm, inv_perm);
     return check_launch("dispatch_small");
   }

@@ -13,6 +13,7 @@
 #include <cstring>
 
 #include "common.h"
+#include "dispatch_small.h"
 
 namespace fs2moe {
 
@@ -591,6 +592,45 @@ __global__ __launch_bounds__(4 * kWave) void router_finish_kernel(
   select_topk<J>(v, lane, t, E, K, score_fn, renorm, topk_idx, topk_w);
 }
 
+// The same for a few tokens in one block, which then goes on to dispatch them (dispatch_small_block:
+// no rows copied): a decode step of a few sequences spends more on starting its kernels than on
+// their work, and this is one start fewer.  A wave takes the tokens wave, wave + 16, ..  Same
+// arithmetic as router_finish_kernel followed by dispatch_small_kernel, so the results are identical.
+constexpr int kFinishDispatchThreads = 1024;
+constexpr int kFinishDispatchTokens = 2 * kFinishDispatchThreads / kWave;
+template <int J>
+__global__ __launch_bounds__(kFinishDispatchThreads) void router_finish_dispatch_kernel(
+    const float* __restrict__ partial, int slices, const float* __restrict__ bias, int T, int E,
+    int K, int score_fn, int renorm, int32_t* topk_idx, float* topk_w, int tile_m, int64_t max_rows,
+    int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv_perm) {
+  extern __shared__ uint32_t s_mem[];
+  __shared__ int32_t s_wave_tot[4];
+  const int lane = lane_id();
+  for (int t = threadIdx.x / kWave; t < T; t += kFinishDispatchThreads / kWave) {  // wave-uniform
+    float p[kMaxSlices][J], b[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+      const int e = lane + 64 * j;
+      b[j] = (bias != nullptr && e < E) ? bias[e] : 0.f;
+#pragma unroll
+      for (int s = 0; s < kMaxSlices; ++s)
+        p[s][j] = (s < slices && e < E) ? partial[((size_t)s * T + t) * E + e] : 0.f;
+    }
+    float v[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+      float sum = p[0][j];
+#pragma unroll
+      for (int s = 1; s < kMaxSlices; ++s) sum += p[s][j];
+      v[j] = sum + b[j];
+    }
+    select_topk<J>(v, lane, t, E, K, score_fn, renorm, topk_idx, topk_w);
+  }
+  __syncthreads();  // the tokens' experts are written and visible to the block
+  dispatch_small_block(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm, s_mem,
+                       s_wave_tot, threadIdx.x, kFinishDispatchThreads);
+}
+
 // ------------------------------------------------------------------------------------ f32 / MFMA
 // The same arrangement for f32 activations on v_mfma_f32_32x32x2_f32 (true f32 products and sums):
 // a 32-token tile per block, 16 waves as 16 / FRP k-groups of FRP waves, wave f of a group owning
@@ -837,7 +877,7 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
                         const void* router, const float* bias, int32_t T, int32_t D, int32_t E,
                         int32_t K, int32_t act_dtype, int32_t score_fn, int32_t renormalize,
                         int32_t* topk_idx, float* topk_w, float* logits, void* workspace,
-                        int64_t workspace_bytes, void* stream) {
+                        int64_t workspace_bytes, DispatchAfterRouter* disp, void* stream) {
   FS2_REQUIRE(x && router && topk_idx && topk_w, "router: null pointer");
   FS2_REQUIRE(xn != x, "router: xn must not alias x");
   FS2_REQUIRE(workspace == nullptr || aligned16(workspace), "router: workspace is not 16-byte aligned");
@@ -926,6 +966,27 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
       if (int rc = check_launch("router_mfma (split)")) return rc;
       const dim3 fgrid((T + 3) / 4), fblock(4 * kWave);
       const int j = (E + 63) / 64;
+      if (disp != nullptr && logits == nullptr && T <= kFinishDispatchTokens) {
+        const size_t dlds = dispatch_small_lds_words(E) * sizeof(uint32_t);
+#define FS2_FINISH_CASE(JJ)                                                                       \
+  case JJ:                                                                                        \
+    hipLaunchKernelGGL((router_finish_dispatch_kernel<JJ>), dim3(1),                                \
+                       dim3(kFinishDispatchThreads), dlds, s,                                     \
+                       partial, slices, bias, T, E, K, score_fn, renormalize, topk_idx, topk_w,   \
+                       disp->tile_m, disp->max_rows, disp->counts, disp->offsets, disp->perm,     \
+                       disp->inv_perm);                                                           \
+    break;
+        switch (j) {
+          FS2_FINISH_CASE(1)
+          FS2_FINISH_CASE(2)
+          FS2_FINISH_CASE(3)
+          FS2_FINISH_CASE(4)
+        }
+#undef FS2_FINISH_CASE
+        if (int rc = check_launch("router_finish_dispatch")) return rc;
+        disp->done = true;
+        return FS2MOE_OK;
+      }
 #define FS2_FINISH_CASE(JJ)                                                                      \
   case JJ:                                                                                       \
     hipLaunchKernelGGL((router_finish_kernel<JJ>), fgrid, fblock, 0, s, partial, slices, bias, T, \
@@ -955,7 +1016,8 @@ extern "C" int fs2moe_router_topk(const void* x, const void* router, const float
                                   float* topk_w, float* logits, void* workspace,
                                   int64_t workspace_bytes, void* stream) {
   return router_entry(x, nullptr, 0.f, nullptr, router, bias, T, D, E, K, act_dtype, score_fn,
-                      renormalize, topk_idx, topk_w, logits, workspace, workspace_bytes, stream);
+                      renormalize, topk_idx, topk_w, logits, workspace, workspace_bytes, nullptr,
+                      stream);
 }
 
 extern "C" int fs2moe_router_topk_norm(const void* x, const void* norm_weight, float norm_eps,
@@ -967,7 +1029,26 @@ extern "C" int fs2moe_router_topk_norm(const void* x, const void* norm_weight, f
   FS2_REQUIRE(xn != nullptr, "router: xn is null");
   FS2_REQUIRE(norm_eps >= 0.f, "router: norm_eps %g is negative", (double)norm_eps);
   return router_entry(x, norm_weight, norm_eps, xn, router, bias, T, D, E, K, act_dtype, score_fn,
-                      renormalize, topk_idx, topk_w, logits, workspace, workspace_bytes, stream);
+                      renormalize, topk_idx, topk_w, logits, workspace, workspace_bytes, nullptr,
+                      stream);
+}
+
+int fs2moe::router_then_dispatch(const void* x, const void* norm_w, float norm_eps, void* xn,
+                                 const void* router, const float* bias, int32_t T, int32_t D,
+                                 int32_t E, int32_t K, int32_t act_dtype, int32_t score_fn,
+                                 int32_t renormalize, int32_t* topk_idx, float* topk_w,
+                                 void* workspace, int64_t workspace_bytes,
+                                 DispatchAfterRouter* disp, void* stream) {
+  FS2_REQUIRE(xn == nullptr || norm_eps >= 0.f, "router: norm_eps %g is negative", (double)norm_eps);
+  if (disp != nullptr) {
+    FS2_REQUIRE(disp->tile_m >= 1 && disp->tile_m <= 1024, "dispatch: tile_m=%d", disp->tile_m);
+    FS2_REQUIRE(disp->counts && disp->offsets && disp->perm && disp->inv_perm,
+                "dispatch: null pointer");
+    disp->done = false;
+  }
+  return router_entry(x, norm_w, norm_eps, xn, router, bias, T, D, E, K, act_dtype, score_fn,
+                      renormalize, topk_idx, topk_w, nullptr, workspace, workspace_bytes, disp,
+                      stream);
 }
 
 // ---- host mirror of the selection -------------------------------------------------------------------

@@ -325,6 +325,10 @@ def test_graphed_forward_replays_match_eager(gpu_device, tokens):
         ("bf16", None, W.RoutingMode("softmax", True, "output"), False, 300),  # fused gather
         ("fp32", None, W.RoutingMode("sigmoid", False, "input"), False, 77),
         ("bf16", "fp8", W.RoutingMode("softmax", True, "output"), False, 40),  # e4m3 weights
+        # a few tokens: the single call dispatches in the router's second kernel, the module's stages separately
+        ("bf16", None, W.RoutingMode("softmax", True, "output"), False, 1),
+        ("bf16", None, W.RoutingMode("softmax", False, "output"), True, 4),
+        ("bf16", "fp8", W.RoutingMode("softmax", True, "output"), False, 3),
     ],
 )
 def test_single_call_entry_point_equals_the_module(gpu_device, dtype, weight_dtype, mode, shared, tokens):
@@ -401,6 +405,11 @@ class _RMSNorm:
         (W.RoutingMode("softmax", True, "output"), False, None),  # rows read through the permutation
         (W.RoutingMode("softmax", True, "output"), False, "fp8"),
         (W.RoutingMode("softmax", True, "output"), False, "prefill"),  # above 4096 tokens
+        # up to 32 bf16 tokens: the router's second kernel also dispatches
+        (W.RoutingMode("softmax", True, "output"), False, "tokens=1"),
+        (W.RoutingMode("softmax", True, "output"), True, "tokens=3"),
+        (W.RoutingMode("sigmoid", True, "output"), False, "tokens=4"),
+        (W.RoutingMode("sigmoid", False, "input"), False, "tokens=2"),  # rows are copied: no merged dispatch
     ],
 )
 def test_pre_norm_and_residual_in_one_call(gpu_device, dtype, mode, shared, weights):
@@ -416,6 +425,8 @@ def test_pre_norm_and_residual_in_one_call(gpu_device, dtype, mode, shared, weig
     tokens = 1300 if shared else 300
     if weights == "prefill":
         tokens, weights = 4200, None
+    elif weights is not None and weights.startswith("tokens="):
+        tokens, weights = int(weights[7:]), None
     spec = W.small_spec(tokens=tokens, model_dim=128, num_experts=8, top_k=2, inner_dim=192, dtype=dtype,
                         weight_dtype=weights, shared=shared, mode=mode, seed=41)
     wl = W.make_workload_from_spec(spec)

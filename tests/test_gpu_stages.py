@@ -73,6 +73,48 @@ def test_router_matches_oracle(gpu_device, dtype, tokens, d, e, k, mode, zipf):
         assert torch.equal(gl, sl) and torch.equal(gw, sw)
 
 
+@pytest.mark.parametrize(
+    "tokens,d,e,k,mode,zipf",
+    [
+        (1, 2048, 128, 8, "softmax_renorm", 1.2),    # the decode step of the benchmark's layer
+        (4, 2048, 128, 8, "softmax_renorm", None),
+        (3, 4096, 8, 2, "softmax_renorm", None),
+        (2, 5120, 16, 1, "sigmoid_renorm", None),
+        (4, 2048, 256, 16, "softmax_plain", 1.0),
+        (3, 8192, 64, 6, "reference", None),
+        (4, 520, 32, 4, "softmax_plain", None),      # 9 chunks of the model dimension over 2 blocks
+        (1, 8, 8, 8, "reference", None),             # one 16-byte chunk per row, K == E
+        (2, 1024, 24, 3, "softmax_renorm", None),
+        (5, 2048, 128, 8, "softmax_renorm", None),
+    ],
+)
+def test_router_of_a_few_tokens(gpu_device, tokens, d, e, k, mode, zipf):
+    """The token counts of a decode step at the model and expert counts of the known layers:
+    against the oracle, and with the normalisation in front."""
+    _say("router, few tokens", tokens, d, e, k, mode)
+    spec = W.small_spec(tokens=tokens, model_dim=d, num_experts=e, top_k=k, inner_dim=8, dtype="bf16",
+                        zipf_s=zipf, mode=MODES[mode], seed=tokens + d)
+    wl = W.make_workload_from_spec(spec, with_weights=False)
+    logits, idx, w = oracle_routing(wl)
+    x = wl.x.reshape(-1, d).bfloat16().to(gpu_device)
+    router = wl.router.bfloat16().to(gpu_device)
+    bias = None if wl.router_bias is None else wl.router_bias.to(gpu_device)
+    score = _abi.SCORE_SOFTMAX if "softmax" in mode else _abi.SCORE_SIGMOID
+    gi, gw, gl = _abi.router_topk(x, router, bias, k, score, spec.mode.renormalize, want_logits=True)
+    np.testing.assert_allclose(gl.cpu().double().numpy(), logits.numpy(), rtol=1e-5, atol=2e-5)
+    assert torch.equal(gi.cpu().long(), idx), "selected experts differ from the oracle"
+    np.testing.assert_allclose(gw.cpu().double().numpy(), w.numpy(), rtol=5e-5, atol=1e-6)
+    # the normalisation in front: the rows, and the routing of those rows
+    g = torch.Generator().manual_seed(d)
+    gamma = (1.0 + 0.3 * torch.randn(d, generator=g)).bfloat16().to(gpu_device)
+    xn, ni, nw, nl = _abi.router_topk_norm(x, gamma, 1e-5, router, bias, k, score,
+                                           spec.mode.renormalize, want_logits=True)
+    want = O.rms_norm(x.cpu(), gamma.cpu(), 1e-5).double()
+    assert bool(((xn.cpu().double() - want).abs() <= 2.0 ** -7 * want.abs()).all())
+    pi, pw, pl = _abi.router_topk(xn, router, bias, k, score, spec.mode.renormalize, want_logits=True)
+    assert torch.equal(ni, pi) and torch.equal(nw, pw) and torch.equal(nl, pl)
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
 @pytest.mark.parametrize(
     "tokens,d,e,k,with_weight",
