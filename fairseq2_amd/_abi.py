@@ -404,7 +404,7 @@ def grouped_swiglu(
     """Returns ``(ye, h)`` for the rows of ``xe`` (rows, D).
 
     ``rows_per_expert``: an upper bound on the rows of any one expert when the caller knows one
-    (the number of tokens is one), else 0; with 1..4 and bf16 weights the products run as streams
+    (the number of tokens is one), else 0; with 1..16 and bf16 weights the products run as streams
     over the weights instead of as GEMM tiles (``fs2moe_grouped_swiglu_rows``).
 
     With ``row_map`` (int32, one entry per row: ``Dispatched.perm``) ``xe`` is the token matrix

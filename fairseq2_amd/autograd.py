@@ -41,7 +41,7 @@ def experts_forward(xe, counts, offsets, wg, wu, wd, e, act=None, rows_per_exper
     """``(ye, g, u)`` of the grouped experts on the rows ``xe``.  Where the expert kernel can, it
     leaves the gate and the up product behind for the backward pass (what autograd would save);
     otherwise ``g`` and ``u`` are None and :func:`experts_backward` computes them again.
-    ``rows_per_expert`` as for :func:`fairseq2_amd._abi.grouped_swiglu`: with a bound of up to 8 the
+    ``rows_per_expert`` as for :func:`fairseq2_amd._abi.grouped_swiglu`: with a bound of up to 16 the
     kernels are those of the inference path at that size (so the values are, too)."""
     if act is not None:
         # a gate activation other than SiLU (experts.py:84-87 takes any module): the module's own
@@ -51,7 +51,7 @@ def experts_forward(xe, counts, offsets, wg, wu, wd, e, act=None, rows_per_exper
         u = _abi.grouped_gemm(xe, wu, _abi.W_IN_OUT, **grp)
         h = (act(g.float()) * u.float()).to(xe.dtype)
         return _abi.grouped_gemm(h, wd, _abi.W_IN_OUT, **grp), g, u
-    if 1 <= rows_per_expert <= 8:
+    if 1 <= rows_per_expert <= 16:
         return _abi.grouped_swiglu(xe, counts, offsets, wg, wu, wd, e, rows_per_expert=rows_per_expert)[0], None, None
     if _abi.keeps_products(xe.shape[1], wd.shape[0] // e, xe.shape[0], xe.dtype):
         ye, _, g, u = _abi.grouped_swiglu_keep(xe, counts, offsets, wg, wu, wd, e)
@@ -132,7 +132,7 @@ def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg, norm_w=None
         idx, w, logits = _abi.router_topk(x, router, cfg["router_bias"], k, score_fn, renorm, want_logits=True)
     disp = _abi.dispatch(idx, w, x, e, tile_m, scale_input, gather=True)
     ye, g, u = experts_forward(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e, cfg.get("activation"),
-                               rows_per_expert=x.shape[0] if x.shape[0] <= 8 else 0)
+                               rows_per_expert=x.shape[0] if x.shape[0] <= 16 else 0)
     base = g_s = u_s = None
     if sg is not None:
         base, g_s, u_s = dense_forward(x, sg, su, sd)

@@ -148,11 +148,11 @@ int forward_impl(bool normed, const void* x_in, const void* norm_weight, float n
                                  scale_input, b.max_rows, b.counts, b.offsets, b.perm, b.inv_perm,
                                  b.xe, b.disp_ws, b.disp_ws_bytes, stream))
       return rc;
-  // (a token takes an expert at most once: with up to 8 tokens no expert has more rows than that)
+  // (a token takes an expert at most once: with up to 16 tokens no expert has more rows than that)
   if (int rc = fs2moe_grouped_swiglu_rows(fused ? x : b.xe, fused ? b.perm : nullptr, b.counts,
                                           b.offsets, w_gate, w_up, w_down, s_gate, s_up, s_down, E,
                                           D, F, b.max_rows, act_dtype, w_dtype, b.h, b.ye,
-                                          T <= 8 ? T : 0, stream))
+                                          T <= 16 ? T : 0, stream))
     return rc;
   const void* base = nullptr;
   if (shared) {

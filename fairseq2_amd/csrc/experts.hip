@@ -400,7 +400,8 @@ static bool dma_offsets_fit(int64_t rows_bound, int D, int F) {
 // The streaming pair for at most `rows_hint` rows per expert: see experts_gemv.h.  Measured on the
 // Qwen3 layer shape (bf16 weights, whole layer, against the GEMM tiles): 1 token 44-47 against 69 us,
 // 2 tokens 52 against 70, 3 tokens 56 against 71, 4 tokens 61 against 72; from 5 rows on the vector
-// ALUs fall behind (8 tokens: 95 against 84 us), so the bound stops at 4.
+// ALUs fall behind (8 tokens: 95 against 84 us), so the bound stops at 4 and the matrix-pipe stream
+// below takes over.
 #ifndef FS2MOE_GEMV_MAX_ROWS
 #define FS2MOE_GEMV_MAX_ROWS 4
 #endif
@@ -444,6 +445,52 @@ static int launch_gemv_pair_r(const void* x, const int32_t* row_map, const Group
   return check_launch("glu_gemv_bf16<down>");
 }
 
+// The same for 5 to 16 rows per expert, on the matrix pipe (glu_gemv16_bf16_kernel).  Whole layer at
+// the Qwen3 shape against the GEMM tiles: 5 tokens 62 against 72 us, 8 tokens 69 against 79, 12 tokens
+// 71 against 81, 16 tokens 82 against 83.  At 3 and 4 rows it ties with the vector-ALU stream (53.5
+// against 52.4 and 56.5 against 57.6 us), at 1 and 2 it loses (48 against 41, 53 against 48: half as
+// many blocks per expert).
+#ifndef FS2MOE_GEMV16_MAX_ROWS
+#define FS2MOE_GEMV16_MAX_ROWS 16
+#endif
+static bool gemv16_applies(int act_dtype, int D, int F, const Groups& g, int rows_hint) {
+  if (act_dtype != FS2MOE_BF16 || g.counts == nullptr || rows_hint <= FS2MOE_GEMV_MAX_ROWS ||
+      rows_hint > FS2MOE_GEMV16_MAX_ROWS)
+    return false;
+  return gemv16::offsets_fit(D, F) && gemv16::fits(D > F ? D : F, rows_hint <= 8 ? 8 : 16);
+}
+
+template <int XR>
+static int launch_gemv16_pair(const void* x, const int32_t* row_map, const Groups& g,
+                              const void* w_gate, const void* w_up, const void* w_down, int D, int F,
+                              void* h, void* y, hipStream_t stream) {
+  using namespace gemv16;
+  auto k1 = glu_gemv16_bf16_kernel<true, XR>;
+  auto k2 = glu_gemv16_bf16_kernel<false, XR>;
+  static bool attr_set = false;  // benign race: setting the attribute is idempotent
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(k1),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS_BYTES) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(k2),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS_BYTES) != hipSuccess) {
+      set_error("experts: cannot reserve %d bytes of LDS", MAX_LDS_BYTES);
+      return FS2MOE_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(k1, dim3((unsigned)((F + COLS - 1) / COLS), (unsigned)g.E), dim3(THREADS),
+                     lds_bytes(D, XR, true), stream, static_cast<const uint16_t*>(x), row_map, D,
+                     static_cast<const uint16_t*>(w_gate), static_cast<const uint16_t*>(w_up),
+                     static_cast<uint16_t*>(h), F, D, F, g.counts, g.offsets);
+  if (int rc = check_launch("glu_gemv16_bf16<gate,up>")) return rc;
+  hipLaunchKernelGGL(k2, dim3((unsigned)((D + COLS - 1) / COLS), (unsigned)g.E), dim3(THREADS),
+                     lds_bytes(F, XR, false), stream, static_cast<const uint16_t*>(h),
+                     static_cast<const int32_t*>(nullptr), F, static_cast<const uint16_t*>(w_down),
+                     static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(y), D, F, D,
+                     g.counts, g.offsets);
+  return check_launch("glu_gemv16_bf16<down>");
+}
+
 // rows_hint: an upper bound on the rows of any one expert when the caller knows one (the number of
 // tokens is one: a token takes an expert at most once), else 0.
 template <int BLAYOUT>
@@ -456,6 +503,10 @@ static int launch_glu(const void* x, const int32_t* row_map, const Groups& g, in
       if (rows_hint <= 1) return launch_gemv_pair_r<1>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
       if (rows_hint <= 2) return launch_gemv_pair_r<2>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
       return launch_gemv_pair_r<4>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
+    }
+    if (gemv16_applies(act_dtype, D, F, g, rows_hint)) {
+      if (rows_hint <= 8) return launch_gemv16_pair<8>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
+      return launch_gemv16_pair<16>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
     }
   }
   if (dma_path_applies(act_dtype, D, F) && dma_offsets_fit(rows_bound, D, F))

@@ -32,6 +32,33 @@ constexpr int MAX_LDS_BYTES = 65536;
 inline bool fits(int K, int R) { return (int64_t)K * R * 2 <= MAX_LDS_BYTES; }
 }  // namespace gemv
 
+// The n-th expert that has rows, -1 when there are fewer (wave-uniform; every wave works it out for
+// itself from the counts, without LDS or a barrier: E <= 256 is four ballots).  A block takes the
+// blockIdx.y-th such expert instead of expert blockIdx.y: blocks of experts without rows would end at
+// once wherever they are, but numbered this way the blocks that work are contiguous in launch order
+// whatever the experts' numbers, and consecutive blocks go to consecutive XCDs.  With the real routing
+// of 12 tokens (24 experts active, scattered over 128) the blocks of the block-per-CU kernel below
+// crowded on some XCDs and its pair of launches took 73 instead of 54 us.
+__device__ __forceinline__ int nth_active_expert(const int32_t* __restrict__ counts, int E, int n) {
+  const int lane = threadIdx.x & 63;
+  int c[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = lane + 64 * j;
+    c[j] = counts[i < E ? i : 0];
+  }
+  int e = -1, seen = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const unsigned long long act = __ballot(lane + 64 * j < E && c[j] > 0);
+    const int before = __popcll(act & ((1ull << lane) - 1ull));
+    const unsigned long long hit = __ballot(((act >> lane) & 1ull) != 0ull && seen + before == n);
+    if (e < 0 && hit != 0ull) e = 64 * j + (int)__builtin_ctzll(hit);
+    seen += __popcll(act);
+  }
+  return e;
+}
+
 // DUAL: C[r, n] = SiLU(A[r] . B0[:, n]) * (A[r] . B1[:, n]); else C[r, n] = A[r] . B0[:, n].
 // A rows are read through row_map when it is given (row r of the expert is A[row_map[offset + r]]).
 // grid: (ceil(N / 64), E).  K a multiple of 4, N a multiple of 8.
@@ -180,6 +207,208 @@ __global__ __launch_bounds__(gemv::threads(R)) void glu_gemv_bf16_kernel(
       }
       if (DUAL) g = silu_f32(g) * u;
       C[(size_t)(off + r0 + r) * ldc + n] = f32_to_bf16_bits(g);
+    }
+  }
+}
+
+
+// ---------------------------------------------------------------------------------------------------
+// The same stream for 5 to 16 rows per expert, with the arithmetic on the matrix pipe and still no
+// LDS transposition of the weights.  v_mfma_f32_16x16x32_bf16 wants, per lane, eight k of ONE
+// channel; a lane's 16-byte load holds eight channels of ONE k.  But the 32 k slots of the
+// instruction are just 32 products summed per (channel, row) pair: which k sits in which slot is
+// free as long as both operands agree.  So a lane (c16 = l % 16, g = l / 16) loads its eight
+// channels 8 c16 .. 8 c16 + 7 at eight k rows (two steps of four consecutive rows), and one byte
+// permute per pair of rows turns that 8 x 8 block of its OWN registers into eight operands, one per
+// channel, each holding the lane's eight k in its eight slots.  MFMA number c of a step then multiplies
+// channels {8 r + c : r = 0..15} (one per lane of a group) with up to 16 rows of the expert over
+// 4 groups x 8 k, and the lane (row m = l % 16, q = l / 16) ends up with channels 8 (4 q + i) + c,
+// i = 0..3.  The rows' operand is what lies in LDS: the 2 x 4 consecutive k of row m.
+//
+// A block owns 128 channels of one expert; its eight waves split K (a step of the block is 128 k
+// rows) and their partial sums meet in LDS in a fixed order ((0+4)+(2+6))+((1+5)+(3+7)).  XR (8 or
+// 16) is how many rows are staged in LDS: a pass takes up to XR rows, an expert with more is walked
+// again.  Rows lie K + 4 elements apart so that the sixteen rows' reads fall into different banks.
+namespace gemv16 {
+constexpr int COLS = 128;     // channels per block: 16 lanes x 8
+constexpr int WAVES = 8, THREADS = WAVES * 64;
+constexpr int KSTEP = WAVES * 16;  // k rows per step of the block: waves x 4 lane groups x 4
+constexpr int MAX_LDS_BYTES = 160 * 1024;
+__host__ __device__ inline int stride(int K) { return K + 4; }
+inline size_t lds_bytes(int K, int XR, bool dual) {
+  const size_t xs = ((size_t)XR * stride(K) + 4) * 2;
+  const size_t red = (size_t)4 * (dual ? 2 : 1) * 32 * 64 * 4;
+  return xs > red ? xs : red;
+}
+inline bool fits(int K, int XR) { return lds_bytes(K, XR, true) <= (size_t)MAX_LDS_BYTES; }
+// (one expert's matrix is addressed with 32-bit byte offsets)
+inline bool offsets_fit(int D, int F) { return (int64_t)D * F * 2 <= 0xffffffffll; }
+}  // namespace gemv16
+
+// Arguments as glu_gemv_bf16_kernel.  grid: (ceil(N / 128), E).  K and N multiples of 8.
+template <bool DUAL, int XR>
+__global__ __launch_bounds__(gemv16::THREADS) void glu_gemv16_bf16_kernel(
+    const uint16_t* __restrict__ A, const int32_t* __restrict__ row_map, int lda,
+    const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1, uint16_t* __restrict__ C,
+    int ldc, int K, int N, const int32_t* __restrict__ counts,
+    const int32_t* __restrict__ offsets) {
+  using namespace gemv16;
+  constexpr int M = DUAL ? 2 : 1;
+  constexpr int PAIRS = DUAL ? 1 : 2;  // pairs of steps per iteration: 16 loads in flight per lane
+  extern __shared__ __attribute__((aligned(16))) uint8_t gemv16_smem[];
+  uint16_t* xs = reinterpret_cast<uint16_t*>(gemv16_smem);  // [XR][K + 4], then 4 zeros
+  float* red = reinterpret_cast<float*>(gemv16_smem);       // [4][M][32][64], after the stream
+
+  const int e = nth_active_expert(counts, (int)gridDim.y, (int)blockIdx.y);
+  if (e < 0) return;
+  const int cnt = counts[e];
+  const int off = offsets[e];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c16 = lane & 15, g = lane >> 4;
+  const int ldx = stride(K);
+  const int col = blockIdx.x * COLS + c16 * 8;
+  const bool col_ok = col < N;  // N is a multiple of 8: the lane's eight channels are in or out together
+  // the expert's matrices as uniform bases, a lane's place in them as a 32-bit byte offset (one
+  // register per address, shared by gate and up)
+  const uint8_t* w0 = reinterpret_cast<const uint8_t*>(B0 + (size_t)e * K * N);
+  const uint8_t* w1 = DUAL ? reinterpret_cast<const uint8_t*>(B1 + (size_t)e * K * N) : w0;
+  const uint32_t lane_col = (uint32_t)(col_ok ? col : 0);
+  const uint16_t* xzero = xs + (size_t)XR * ldx;
+  const uint16_t* xrow = xs + (size_t)c16 * ldx;  // row m = c16 of the pass, if it is staged
+  const bool row_ok = c16 < XR;
+
+  for (int r0 = 0; r0 < cnt; r0 += XR) {
+    // ---- the pass's rows -> LDS (rows past the expert's count as zeros) ---------------------------
+    if (r0 > 0) __syncthreads();  // the previous pass's sums have left LDS
+    // (a row per group of threads, so that the row's place is looked up once and a thread's loads
+    // are all in flight together; K is a multiple of 8 here: 16-byte pieces)
+    {
+      constexpr int TPR = THREADS / XR, INFLIGHT = 4;
+      const int r = tid / TPR, c0 = tid - r * TPR;
+      const int kchunks = K / 8;
+      const bool has = r0 + r < cnt;
+      size_t src = 0;
+      if (has) {
+        const int row = off + r0 + r;
+        src = (size_t)(row_map != nullptr ? row_map[row] : row) * lda;
+      }
+      for (int cb = c0; cb < kchunks; cb += TPR * INFLIGHT) {
+        u32x4 v[INFLIGHT];
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u) {
+          const int c = cb + u * TPR;
+          v[u] = *reinterpret_cast<const u32x4*>(A + src + 8 * (c < kchunks ? c : 0));
+        }
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u) {
+          const int c = cb + u * TPR;
+          if (c >= kchunks) continue;
+          if (!has) v[u] = u32x4{0u, 0u, 0u, 0u};
+          u32x2* dst = reinterpret_cast<u32x2*>(xs + (size_t)r * ldx + 8 * c);  // 8-byte aligned
+          dst[0] = u32x2{v[u][0], v[u][1]};
+          dst[1] = u32x2{v[u][2], v[u][3]};
+        }
+      }
+    }
+    if (tid < 4) xs[(size_t)XR * ldx + tid] = 0;
+    __syncthreads();
+
+    // ---- the stream over K --------------------------------------------------------------------------
+    f32x4 acc[M][8];
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+      for (int c = 0; c < 8; ++c) acc[m][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int kb0 = 0; kb0 < K; kb0 += 2 * PAIRS * KSTEP) {
+      u32x4 wq[2 * PAIRS][M][4];
+      u32x2 xq[2 * PAIRS];
+#pragma unroll
+      for (int s = 0; s < 2 * PAIRS; ++s) {
+        const int k0 = kb0 + s * KSTEP + wave * 16 + g * 4;
+        const bool k_ok = k0 < K;  // K is a multiple of 4: the lane's four rows are in or out together
+        const int kk = k_ok ? k0 : 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t at = ((uint32_t)(kk + j) * (uint32_t)N + lane_col) * 2u;
+          wq[s][0][j] = *reinterpret_cast<const u32x4*>(w0 + at);
+          if (DUAL) wq[s][M - 1][j] = *reinterpret_cast<const u32x4*>(w1 + at);
+        }
+        // (k rows past K meet zeros: chosen by address, a select on the value would become a branch)
+        xq[s] = *reinterpret_cast<const u32x2*>(k_ok && row_ok ? xrow + k0 : xzero);
+      }
+      // (without the fence the compiler moves every load down to its first use and waits for each
+      // one there: one round trip per load instead of one per iteration)
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int p = 0; p < PAIRS; ++p) {
+        const u32x4 xo = {xq[2 * p][0], xq[2 * p][1], xq[2 * p + 1][0], xq[2 * p + 1][1]};
+        const bf16x8 xop = __builtin_bit_cast(bf16x8, xo);
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+          for (int c = 0; c < 8; ++c) {
+            // channel c of the lane: the low (c even) or high (c odd) half of dword c / 2 of each row
+            const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+            const u32x4(&a)[4] = wq[2 * p][m];
+            const u32x4(&b)[4] = wq[2 * p + 1][m];
+            const u32x4 wo = {__builtin_amdgcn_perm(a[1][c >> 1], a[0][c >> 1], sel),
+                              __builtin_amdgcn_perm(a[3][c >> 1], a[2][c >> 1], sel),
+                              __builtin_amdgcn_perm(b[1][c >> 1], b[0][c >> 1], sel),
+                              __builtin_amdgcn_perm(b[3][c >> 1], b[2][c >> 1], sel)};
+            acc[m][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wo), xop,
+                                                                 acc[m][c], 0, 0, 0);
+            // (operands are formed four channels ahead at most: formed all at once they cost 64
+            // registers and the kernel spills)
+            if ((c & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+          }
+      }
+    }
+
+    // ---- the waves' sums meet in LDS: (w + 4) onto w, then (w + 2) onto w, then 1 onto 0 ------------
+    __syncthreads();  // every wave is done reading the rows: the sums take their place
+#pragma unroll
+    for (int half = 4; half >= 1; half >>= 1) {
+      // (one address register per wave and constant offsets from it)
+      if (wave >= half && wave < 2 * half) {
+        float* rp = red + (wave - half) * (M * 32 * 64) + lane;
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+          for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) rp[(m * 32 + c * 4 + i) * 64] = acc[m][c][i];
+      }
+      __syncthreads();
+      if (wave < half) {
+        const float* rp = red + wave * (M * 32 * 64) + lane;
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+          for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[m][c][i] += rp[(m * 32 + c * 4 + i) * 64];
+      }
+      if (half > 1) __syncthreads();
+    }
+    // ---- wave 0: row m = l % 16, channels 8 (4 q + i) + c ---------------------------------------------
+    if (wave == 0 && r0 + c16 < cnt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = blockIdx.x * COLS + (4 * g + i) * 8;
+        if (n >= N) continue;
+        u32x4 o;
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          float v0 = acc[0][2 * h][i], v1 = acc[0][2 * h + 1][i];
+          if (DUAL) {
+            v0 = silu_f32(v0) * acc[M - 1][2 * h][i];
+            v1 = silu_f32(v1) * acc[M - 1][2 * h + 1][i];
+          }
+          o[h] = (uint32_t)f32_to_bf16_bits(v0) | ((uint32_t)f32_to_bf16_bits(v1) << 16);
+        }
+        *reinterpret_cast<u32x4*>(C + (size_t)(off + r0 + c16) * ldc + n) = o;
+      }
     }
   }
 }

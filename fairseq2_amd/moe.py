@@ -222,7 +222,7 @@ class GroupedExpertNetwork(ExpertNetwork):
     ) -> Tensor:
         """Runs every expert on its block of rows of ``xe`` (rows, D); with ``row_map``, row ``r``
         is ``xe[row_map[r]]`` and ``xe`` is the token matrix.  ``rows_per_expert``: an upper bound
-        on any expert's rows when the caller knows one (the number of tokens is one), else 0; up to 8
+        on any expert's rows when the caller knows one (the number of tokens is one), else 0; up to 16
         the bf16 experts run as streams over their weights.  Inference only (the training paths are
         :meth:`forward` and the layer's)."""
         _require_forward_only(xe, self.gate_proj, self.inner_proj, self.output_proj)
@@ -271,11 +271,11 @@ class GroupedExpertNetwork(ExpertNetwork):
 
             ye = GroupedExpertsFunction.apply(
                 x.reshape(e * n, d).contiguous(), counts, offsets, *params, e,
-                None if self.has_fused_gate else self.activation, n if n <= 8 else 0)
+                None if self.has_fused_gate else self.activation, n if n <= 16 else 0)
             return ye.view(e, n, d)
         # (every expert has exactly n rows: a bound the library can use when it is small)
         return self.forward_rows(x.reshape(e * n, d).contiguous(), counts, offsets,
-                                 rows_per_expert=n if n <= 8 else 0).view(e, n, d)
+                                 rows_per_expert=n if n <= 16 else 0).view(e, n, d)
 
     def _uniform_groups(self, n: int, device: torch.device) -> tuple[Tensor, Tensor]:
         """counts / offsets of ``n`` rows for every expert, built once per (n, device) so that the
@@ -637,9 +637,9 @@ class MoE(FeedForwardNetwork):
         disp = _abi.dispatch(
             idx, w, x, ex.num_local_experts, self.tile_m, scale_input, gather=not fused
         )
-        # a token takes an expert at most once: with up to 8 tokens no expert has more rows than that
+        # a token takes an expert at most once: with up to 16 tokens no expert has more rows than that
         # (what the whole-layer call passes on as well)
-        hint = dict(rows_per_expert=x.shape[0]) if isinstance(ex, GroupedExpertNetwork) and x.shape[0] <= 8 else {}
+        hint = dict(rows_per_expert=x.shape[0]) if isinstance(ex, GroupedExpertNetwork) and x.shape[0] <= 16 else {}
         if fused:
             ye = ex.forward_rows(x, disp.counts, disp.offsets, row_map=disp.perm, **hint)
         else:

@@ -163,8 +163,9 @@ int fs2moe_grouped_swiglu(const void* xe, const int32_t* row_map, const int32_t*
  * (rows_per_expert; 0: no bound known, then this is fs2moe_grouped_swiglu).  The number of tokens is
  * such a bound (torch.topk of moe.py:113 gives a token an expert at most once), which is what a
  * decode step of a few sequences (generation/: one token per sequence and step) has to offer: with
- * a bound of 1..4 and bf16 weights the two products run as streams over the active experts' weights
- * on the vector ALUs (no LDS tiles, no matrix pipe) instead of as GEMM tiles (larger bounds: as 0).  Same arguments and
+ * a bound of 1..16 and bf16 weights the two products run as streams over the active experts' weights
+ * (no LDS tiles; up to 4 rows on the vector ALUs, 5..16 on the matrix pipe) instead of as GEMM tiles
+ * (larger bounds: as 0).  Same arguments and
  * results (to the order of f32 additions) otherwise; a count above the bound is still computed
  * correctly, only slowly.
  */

@@ -331,12 +331,21 @@ def test_grouped_swiglu_matches_oracle(gpu_device, dtype, rows_per_expert, d, f)
         (8, [(3 * i) % 9 for i in range(128)], 64, 64),
         (4, [9, 4, 13, 0, 1], 128, 64),               # counts above the bound: walked again, still right
         (4, [4, 2], 8192, 64),                        # the longest K whose four rows fit LDS
+        # 5 to 16 rows: the same stream with the arithmetic on the matrix pipe
+        (16, [16, 9, 0, 12, 1, 5], 2048, 768),       # the Qwen3 shape
+        (12, [12, 3, 7], 72, 40),                     # K and N off the kernel's steps
+        (5, [5, 0, 2, 5], 256, 136),
+        (16, [16, 2], 5112, 64),                      # the longest K whose sixteen rows fit LDS
+        (8, [8, 1], 8192, 64),                        # eight rows staged
+        (8, [20, 8, 9], 128, 136),                    # counts above the bound
+        (16, [33, 16, 0, 17], 64, 200),
     ],
 )
 def test_grouped_swiglu_with_a_bound_on_the_rows_per_expert(gpu_device, bound, rows_per_expert, d, f):
     """``fs2moe_grouped_swiglu_rows``: with a bound of 1..4 rows per expert and bf16 weights the two
-    products stream the weights through the vector ALUs (larger bounds take the GEMM kernels).  Each
-    expert against the oracle's SwiGLU in f64; rows read through a map give the same bits."""
+    products stream the weights through the vector ALUs, with 5..16 through the matrix pipe (larger
+    bounds take the GEMM kernels).  Each expert against the oracle's SwiGLU in f64; rows read
+    through a map give the same bits."""
     _say("grouped_swiglu_rows", bound, rows_per_expert[:8], d, f)
     counts, offsets, xe, wg, wu, wd = _expert_case("bf16", rows_per_expert, d, f, seed=bound + d + f)
     e = len(rows_per_expert)
@@ -365,8 +374,8 @@ def test_grouped_swiglu_with_a_bound_on_the_rows_per_expert(gpu_device, bound, r
     for ex in range(e):
         lo, n = int(offsets[ex]), int(counts[ex])
         assert torch.equal(ye2[lo : lo + n], ye[lo : lo + n]) and torch.equal(h2[lo : lo + n], h[lo : lo + n])
-    # bounds outside 1..4 take the other kernels; a negative bound is refused
-    ye3, _ = _abi.grouped_swiglu(xe.to(bf).to(dev), *args, rows_per_expert=9)
+    # bounds outside 1..16 take the other kernels; a negative bound is refused
+    ye3, _ = _abi.grouped_swiglu(xe.to(bf).to(dev), *args, rows_per_expert=17)
     ye4, _ = _abi.grouped_swiglu(xe.to(bf).to(dev), *args)
     for ex in range(e):
         lo, n = int(offsets[ex]), int(counts[ex])
