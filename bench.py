@@ -104,6 +104,8 @@ def time_stages(module, x, reps: int):
     # as in MoE._stages: unscaled rows are read through the permutation by the first GEMM
     fused = (not scale_input) and hasattr(ex, "fuses_gather") and ex.fuses_gather(x.dtype)
     names = ["router", "dispatch", "experts"] + (["shared"] if module.shared_expert else []) + ["combine"]
+    # as in MoE._stages: a token takes an expert at most once, a bound the expert stage uses when small
+    bound = x.shape[0] if x.shape[0] <= 16 else 0
     tot = {n: 0.0 for n in names}
     tot["dispatch_with_gather"] = 0.0
     ev = lambda: torch.cuda.Event(enable_timing=True)
@@ -131,9 +133,11 @@ def time_stages(module, x, reps: int):
             idx, w, x, ex.num_local_experts, module.tile_m, scale_input, gather=not fused
         ))
         if fused:
-            ye, spans["experts"] = timed(lambda: ex.forward_rows(x, disp.counts, disp.offsets, row_map=disp.perm))
+            ye, spans["experts"] = timed(lambda: ex.forward_rows(x, disp.counts, disp.offsets, row_map=disp.perm,
+                                                                 rows_per_expert=bound))
         else:
-            ye, spans["experts"] = timed(lambda: ex.forward_rows(disp.xe, disp.counts, disp.offsets))
+            ye, spans["experts"] = timed(lambda: ex.forward_rows(disp.xe, disp.counts, disp.offsets,
+                                                                 rows_per_expert=bound))
         base = None
         if module.shared_expert is not None:
             base, spans["shared"] = timed(lambda: module.shared_expert(x))
@@ -387,6 +391,10 @@ def main() -> int:
         kernel = "glu_gemm_%s_dma_kernel<gate,up> + <down> (fs2moe_grouped_swiglu)" % spec.dtype
     if spec.dtype == "fp32":
         kernel = "glu_gemm_f32_kernel<gate,up> + <down> (fs2moe_grouped_swiglu)"
+    if spec.dtype == "bf16" and spec.weight_dtype == "bf16" and spec.num_tokens <= 16:
+        # a few rows per expert: the weights are streamed without LDS tiles
+        kernel = "%s<gate,up> + <down> (fs2moe_grouped_swiglu_rows)" % (
+            "glu_gemv_bf16_kernel" if spec.num_tokens <= 4 else "glu_gemv16_bf16_kernel")
     if experts_hbm_bound:
         achieved = work["experts"]["bytes"] / (exp_ms * 1e-3) / 1e9
         roofline = {

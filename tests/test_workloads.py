@@ -27,6 +27,8 @@ def _counts(name):
         ("qwen3_30b_a3b", [8138, 7691, 6939, 6074, 5198], dict(median=11, empty=17, le8=59)),
         ("llama4_scout", [552, 546, 538, 536, 534], dict(min=486)),
         ("qwen3_decode_fp8", [64, 60, 55, 47, 46], dict(active=44)),
+        ("qwen3_decode_bf16_1", [1, 1, 1, 1, 1], dict(active=8)),
+        ("qwen3_decode_bf16_8", [8, 8, 8, 6, 5], dict(active=20)),
     ],
 )
 def test_routing_statistics(name, top5, extra):

@@ -106,6 +106,15 @@ SPECS: dict[str, WorkloadSpec] = {
         "qwen3_decode_fp8", 4, 64, 1, 2048, 128, 8, 768, "bf16", "fp8", 1.2, False,
         RoutingMode("softmax", True, "output"),
     ),
+    # decode steps of one and of eight sequences with the weights as the reference holds them
+    "qwen3_decode_bf16_1": WorkloadSpec(
+        "qwen3_decode_bf16_1", 5, 1, 1, 2048, 128, 8, 768, "bf16", "bf16", 1.2, False,
+        RoutingMode("softmax", True, "output"),
+    ),
+    "qwen3_decode_bf16_8": WorkloadSpec(
+        "qwen3_decode_bf16_8", 6, 8, 1, 2048, 128, 8, 768, "bf16", "bf16", 1.2, False,
+        RoutingMode("softmax", True, "output"),
+    ),
 }
 
 FP8_MAX = 448.0  # largest finite OCP e4m3fn value
