@@ -397,12 +397,21 @@ __global__ __launch_bounds__(rmfma::Shape<NF>::THREADS) void router_mfma_kernel(
   const int t0 = blockIdx.x * BT;
   uint16_t* sX = reinterpret_cast<uint16_t*>(smem + group * S::GROUP_BYTES);
   uint16_t* sR = sX + BT * LDX;
-  if constexpr (!SPLIT) {
-    if (xn != nullptr) {
-      rms_norm_block_rows<uint16_t>(x, norm_w, norm_eps, xn, t0, T - t0 < BT ? T - t0 : BT, D, 0, D);
-      __syncthreads();  // the block's rows of xn are written and visible to all its waves
-      x = xn;
+  if (xn != nullptr) {
+    // the columns this block goes on to read: all of them, or (SPLIT, a single token tile: the host
+    // sends more tiles than that through rms_norm_kernel first) the chunks of its share, which the
+    // blocks of the tile write between them
+    int k_lo = 0, k_hi = D;
+    if constexpr (SPLIT) {
+      const int nk_all = (D + BK - 1) / BK;
+      const int share = (nk_all + (int)gridDim.y - 1) / (int)gridDim.y;
+      k_lo = (int)blockIdx.y * share * BK;
+      k_hi = k_lo + share * BK < D ? k_lo + share * BK : D;
     }
+    if (k_lo < k_hi)
+      rms_norm_block_rows<uint16_t>(x, norm_w, norm_eps, xn, t0, T - t0 < BT ? T - t0 : BT, D, k_lo, k_hi);
+    __syncthreads();  // the block's part of xn is written and visible to all its waves
+    x = xn;
   }
 
   f32x16 acc[NF];
@@ -892,7 +901,11 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
               act_dtype);
   if (T == 0) return FS2MOE_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (xn != nullptr && T <= kNormAloneMaxTokens) {
+  // (a single token tile of the bf16 MFMA router normalises in its own blocks, also when several
+  // blocks share the tile: one launch fewer for a decode step)
+  const bool one_tile = act_dtype == FS2MOE_BF16 && T <= rmfma::BT && D % 8 == 0 && E % 8 == 0 &&
+                        aligned16(x) && aligned16(router) && aligned16(xn);
+  if (xn != nullptr && T <= kNormAloneMaxTokens && !one_tile) {
     // few token blocks: normalise with the whole chip first, then route xn as it is
     dim3 grid((T + kNormRows - 1) / kNormRows), block(kNormRows * kWave);
     if (act_dtype == FS2MOE_F32)
@@ -957,7 +970,8 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
     const dim3 threads(E <= 128 ? rmfma::Shape<1>::THREADS : rmfma::Shape<2>::THREADS);
     const int lds = E <= 128 ? rmfma::Shape<1>::SMEM_BYTES : rmfma::Shape<2>::SMEM_BYTES;
     if (slices > 1 && workspace != nullptr && workspace_bytes >= (int64_t)slices * T * E * 4) {
-      // (the rows were normalised by the kernel in front: T is within kNormAloneMaxTokens)
+      // (several tiles were normalised by the kernel in front, T being within kNormAloneMaxTokens;
+      // a single tile is normalised by its blocks, each the columns it reads)
       static_assert(256 * rmfma::BT / 2 <= kNormAloneMaxTokens, "split tiles are normalised in front");
       float* partial = static_cast<float*>(workspace);
       grid.y = slices;

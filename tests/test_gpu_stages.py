@@ -113,6 +113,11 @@ def test_router_of_a_few_tokens(gpu_device, tokens, d, e, k, mode, zipf):
     assert bool(((xn.cpu().double() - want).abs() <= 2.0 ** -7 * want.abs()).all())
     pi, pw, pl = _abi.router_topk(xn, router, bias, k, score, spec.mode.renormalize, want_logits=True)
     assert torch.equal(ni, pi) and torch.equal(nw, pw) and torch.equal(nl, pl)
+    # up to 32 tokens the router's blocks normalise the columns they read; more tokens go through a
+    # kernel in front: the same rows among 40 come out with the same bits
+    many = torch.cat([x, x.flip(0).repeat(40, 1)[: 40 - tokens]])
+    xn40 = _abi.router_topk_norm(many, gamma, 1e-5, router, bias, k, score, spec.mode.renormalize)[0]
+    assert torch.equal(xn40[:tokens], xn)
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
