@@ -246,8 +246,11 @@ inline bool offsets_fit(int D, int F) { return (int64_t)D * F * 2 <= 0xffffffffl
 }  // namespace gemv16
 
 // Arguments as glu_gemv_bf16_kernel.  grid: (ceil(N / 128), E).  K and N multiples of 8.
+// (The second launch bound is waves per SIMD: the single product is held to 128 registers so that
+// two blocks share a CU -- the down projection of 20 active experts is 320 blocks, which at one block
+// per CU ran as a full round and a quarter-full one: 4 us of 75 at 8 tokens.)
 template <bool DUAL, int XR>
-__global__ __launch_bounds__(gemv16::THREADS) void glu_gemv16_bf16_kernel(
+__global__ __launch_bounds__(gemv16::THREADS, DUAL ? 2 : 4) void glu_gemv16_bf16_kernel(
     const uint16_t* __restrict__ A, const int32_t* __restrict__ row_map, int lda,
     const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1, uint16_t* __restrict__ C,
     int ldc, int K, int N, const int32_t* __restrict__ counts,
