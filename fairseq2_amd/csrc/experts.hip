@@ -446,8 +446,8 @@ static int launch_gemv_pair_r(const void* x, const int32_t* row_map, const Group
 }
 
 // The same for 5 to 16 rows per expert, on the matrix pipe (glu_gemv16_bf16_kernel).  Whole layer at
-// the Qwen3 shape against the GEMM tiles: 5 tokens 62 against 72 us, 8 tokens 69 against 79, 12 tokens
-// 71 against 81, 16 tokens 82 against 83.  At 3 and 4 rows it ties with the vector-ALU stream (53.5
+// the Qwen3 shape against the GEMM tiles: 5 tokens 57 against 72 us, 8 tokens 69-71 against 79, 12
+// tokens 71 against 81, 16 tokens 78 against 83.  At 3 and 4 rows it ties with the vector-ALU stream (53.5
 // against 52.4 and 56.5 against 57.6 us), at 1 and 2 it loses (48 against 41, 53 against 48: half as
 // many blocks per expert).
 #ifndef FS2MOE_GEMV16_MAX_ROWS
