@@ -457,7 +457,12 @@ static bool gemv16_applies(int act_dtype, int D, int F, const Groups& g, int row
   if (act_dtype != FS2MOE_BF16 || g.counts == nullptr || rows_hint <= FS2MOE_GEMV_MAX_ROWS ||
       rows_hint > FS2MOE_GEMV16_MAX_ROWS)
     return false;
-  return gemv16::offsets_fit(D, F) && gemv16::fits(D > F ? D : F, rows_hint <= 8 ? 8 : 16);
+  return gemv16::offsets_fit(D, F) && gemv16::fits(D > F ? D : F, 8);
+}
+// rows staged per pass: 16 when the bound asks for it and rows that long fit LDS, else 8 (an expert
+// with more rows is walked again)
+static int gemv16_rows(int D, int F, int rows_hint) {
+  return rows_hint > 8 && gemv16::fits(D > F ? D : F, 16) ? 16 : 8;
 }
 
 template <int XR>
@@ -505,7 +510,8 @@ static int launch_glu(const void* x, const int32_t* row_map, const Groups& g, in
       return launch_gemv_pair_r<4>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
     }
     if (gemv16_applies(act_dtype, D, F, g, rows_hint)) {
-      if (rows_hint <= 8) return launch_gemv16_pair<8>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
+      if (gemv16_rows(D, F, rows_hint) == 8)
+        return launch_gemv16_pair<8>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
       return launch_gemv16_pair<16>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
     }
   }

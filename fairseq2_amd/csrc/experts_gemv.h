@@ -28,7 +28,7 @@ constexpr int COLS = 64;          // channels per block
 // waves (with four, one token took 47 instead of 44 us and four tokens 71 instead of 61)
 constexpr int waves(int R) { return 8; }
 constexpr int threads(int R) { return 64 * waves(R); }
-constexpr int MAX_LDS_BYTES = 65536;
+constexpr int MAX_LDS_BYTES = 144 * 1024;  // (160 KB less the kernel's own partial sums, 16 KB at most)
 inline bool fits(int K, int R) { return (int64_t)K * R * 2 <= MAX_LDS_BYTES; }
 }  // namespace gemv
 

@@ -335,13 +335,15 @@ def test_grouped_swiglu_matches_oracle(gpu_device, dtype, rows_per_expert, d, f)
         (8, [8, 5, 0, 7, 1, 8, 3], 320, 192),
         (8, [(3 * i) % 9 for i in range(128)], 64, 64),
         (4, [9, 4, 13, 0, 1], 128, 64),               # counts above the bound: walked again, still right
-        (4, [4, 2], 8192, 64),                        # the longest K whose four rows fit LDS
+        (4, [4, 2], 8192, 64),
+        (4, [4, 1], 18432, 64),                       # the longest K whose four rows fit LDS
         # 5 to 16 rows: the same stream with the arithmetic on the matrix pipe
         (16, [16, 9, 0, 12, 1, 5], 2048, 768),       # the Qwen3 shape
         (12, [12, 3, 7], 72, 40),                     # K and N off the kernel's steps
         (5, [5, 0, 2, 5], 256, 136),
         (16, [16, 2], 5112, 64),                      # the longest K whose sixteen rows fit LDS
         (8, [8, 1], 8192, 64),                        # eight rows staged
+        (16, [16, 2, 9], 8192, 64),                   # sixteen such rows do not fit: eight at a time
         (8, [20, 8, 9], 128, 136),                    # counts above the bound
         (16, [33, 16, 0, 17], 64, 200),
     ],
