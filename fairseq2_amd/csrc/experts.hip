@@ -496,6 +496,25 @@ static int launch_gemv16_pair(const void* x, const int32_t* row_map, const Group
   return check_launch("glu_gemv16_bf16<down>");
 }
 
+// The dense SwiGLU (the shared expert, weights (N, K)) of up to 16 bf16 rows: dense_gemv_bf16_kernel.
+// Llama-4 Scout's shared expert (D 5120, F 8192): 1 token 172 us on the GEMM tiles.
+static bool dense_gemv_applies(int act_dtype, const Groups& g, int64_t rows) {
+  return act_dtype == FS2MOE_BF16 && g.counts == nullptr && rows >= 1 && rows <= dgemv::MAX_ROWS;
+}
+static int launch_dense_gemv_pair(const void* x, int T, const void* w_gate, const void* w_up,
+                                  const void* w_down, int D, int F, void* h, void* y,
+                                  hipStream_t stream) {
+  using namespace dgemv;
+  hipLaunchKernelGGL(dense_gemv_bf16_kernel<true>, dim3((unsigned)((F + 15) / 16)), dim3(THREADS), 0,
+                     stream, static_cast<const uint16_t*>(x), D, static_cast<const uint16_t*>(w_gate),
+                     static_cast<const uint16_t*>(w_up), static_cast<uint16_t*>(h), F, D, F, T);
+  if (int rc = check_launch("dense_gemv_bf16<gate,up>")) return rc;
+  hipLaunchKernelGGL(dense_gemv_bf16_kernel<false>, dim3((unsigned)((D + 15) / 16)), dim3(THREADS), 0,
+                     stream, static_cast<const uint16_t*>(h), F, static_cast<const uint16_t*>(w_down),
+                     static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(y), D, F, D, T);
+  return check_launch("dense_gemv_bf16<down>");
+}
+
 // rows_hint: an upper bound on the rows of any one expert when the caller knows one (the number of
 // tokens is one: a token takes an expert at most once), else 0.
 template <int BLAYOUT>
@@ -503,6 +522,10 @@ static int launch_glu(const void* x, const int32_t* row_map, const Groups& g, in
                       const void* w_gate, const void* w_up, const void* w_down, int D, int F,
                       int act_dtype, void* h, void* y, hipStream_t stream, int rows_hint = 0) {
   const int groups = g.counts ? g.E : 0;
+  if constexpr (BLAYOUT == FS2MOE_W_OUT_IN) {
+    if (row_map == nullptr && dense_gemv_applies(act_dtype, g, rows_bound))
+      return launch_dense_gemv_pair(x, (int)rows_bound, w_gate, w_up, w_down, D, F, h, y, stream);
+  }
   if constexpr (BLAYOUT == FS2MOE_W_IN_OUT) {
     if (gemv_applies(act_dtype, D, F, g, rows_hint)) {
       if (rows_hint <= 1) return launch_gemv_pair_r<1>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);

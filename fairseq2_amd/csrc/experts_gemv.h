@@ -416,4 +416,88 @@ __global__ __launch_bounds__(gemv16::THREADS, DUAL ? 2 : 4) void glu_gemv16_bf16
   }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The shared expert (a dense SwiGLU, weights as nn.Linear holds them: (N, K) with K contiguous) for
+// up to 16 rows: at a decode step its three matrices are streamed once like an expert's, and the
+// GEMM tiles make that a chain of K / 64 round trips per tile (Llama-4 Scout, one token: 172 us for
+// 252 MB).  Here 16 bytes of a weight row ARE eight k of one channel, which is what
+// v_mfma_f32_16x16x32_bf16 takes from lane (n = l % 16, g = l / 16) as it stands; the matching lane
+// (m = l % 16, g) loads the same eight k of row m straight from memory (the rows stay in L2; a row
+// the call does not have repeats the last one, its results are not stored).  A block owns 16
+// channels, its eight waves split K in steps of 32 and add their sums in LDS in ascending order.
+namespace dgemv {
+constexpr int WAVES = 8, THREADS = WAVES * 64;
+constexpr int U = 8;  // steps of 32 k a wave has in flight
+constexpr int MAX_ROWS = 16;
+}  // namespace dgemv
+
+// DUAL: C[r, n] = SiLU(A[r] . B0[n]) * (A[r] . B1[n]); else C[r, n] = A[r] . B0[n].
+// A [T][lda], B0/B1 [N][K], C [T][ldc]; T <= 16; K and N multiples of 8.  grid: ceil(N / 16).
+template <bool DUAL>
+__global__ __launch_bounds__(dgemv::THREADS) void dense_gemv_bf16_kernel(
+    const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ B0,
+    const uint16_t* __restrict__ B1, uint16_t* __restrict__ C, int ldc, int K, int N, int T) {
+  using namespace dgemv;
+  constexpr int M = DUAL ? 2 : 1;
+  __shared__ f32x4 red[WAVES][M][64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int n = n0 + r16 < N ? n0 + r16 : N - 1;  // a channel past N repeats the last one: not stored
+  const int row = r16 < T ? r16 : T - 1;
+  const uint16_t* w0 = B0 + (size_t)n * K;
+  const uint16_t* w1 = DUAL ? B1 + (size_t)n * K : w0;
+  const uint16_t* xr = A + (size_t)row * lda;
+  f32x4 acc[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) acc[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // step s of the block is the 32 k from 32 s; wave w takes the steps w, w + 8, ..
+  for (int s0 = wave; s0 * 32 < K; s0 += WAVES * U) {
+    u32x4 wq[U][M], xq[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = (s0 + u * WAVES) * 32 + g * 8;
+      const int kk = k < K ? k : 0;  // K is a multiple of 8: the lane's eight k are in or out together
+      wq[u][0] = *reinterpret_cast<const u32x4*>(w0 + kk);
+      if (DUAL) wq[u][M - 1] = *reinterpret_cast<const u32x4*>(w1 + kk);
+      xq[u] = *reinterpret_cast<const u32x4*>(xr + kk);
+    }
+    // (all the loads are issued before the first is waited for)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = (s0 + u * WAVES) * 32 + g * 8;
+      u32x4 xv = xq[u];
+      if (k >= K) xv = u32x4{0u, 0u, 0u, 0u};
+      const bf16x8 xop = __builtin_bit_cast(bf16x8, xv);
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+        acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wq[u][m]), xop,
+                                                         acc[m], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < M; ++m) red[wave][m][lane] = acc[m];
+  __syncthreads();
+  if (wave != 0) return;
+  // lane (row m = l % 16, q = l / 16) holds channels n0 + 4 q + i, i = 0..3
+  f32x4 sum[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    sum[m] = red[0][m][lane];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) sum[m] += red[w][m][lane];
+  }
+  const int nc = n0 + 4 * g;
+  if (r16 < T && nc < N) {  // N is a multiple of 8: four channels are in or out together
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = DUAL ? silu_f32(sum[0][i]) * sum[M - 1][i] : sum[0][i];
+    u32x2 o = {(uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16),
+               (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16)};
+    *reinterpret_cast<u32x2*>(C + (size_t)r16 * ldc + nc) = o;
+  }
+}
+
 }  // namespace fs2moe

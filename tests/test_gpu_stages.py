@@ -469,7 +469,14 @@ def test_grouped_swiglu_fp8_row_map_equals_gathered_rows(gpu_device, t, d, e, k,
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
-@pytest.mark.parametrize("t,d,f", [(200, 128, 256), (37, 72, 40), (1, 64, 64), (600, 192, 320)])
+@pytest.mark.parametrize(
+    "t,d,f",
+    [
+        (200, 128, 256), (37, 72, 40), (1, 64, 64), (600, 192, 320),
+        # up to 16 bf16 rows stream the weights (K off the 32-wide steps, N off the 16-channel blocks)
+        (1, 5120, 1024), (3, 72, 40), (8, 2048, 768), (16, 1000, 200), (16, 8, 8), (17, 256, 128),
+    ],
+)
 def test_dense_swiglu_matches_oracle(gpu_device, dtype, t, d, f):
     _say("dense_swiglu", dtype, t, d, f)
     g = torch.Generator().manual_seed(t)
