@@ -184,6 +184,8 @@ int fs2moe_grouped_swiglu_fuses_gather(int32_t D, int32_t F, int32_t act_dtype, 
  *   y = (SiLU(x @ Wg^T) * (x @ Wu^T)) @ Wd^T  with nn.Linear-oriented weights.
  * Replaces moe.py:143-145 -> ffn.py:374-395 (three F.linear and the SiLU gate).
  *   x [T, D]   w_gate, w_up [F, D]   w_down [D, F]   h [T, F] scratch   y [T, D] (out)
+ * Up to 16 bf16 rows (a decode step) run as a stream over the three matrices instead of as GEMM
+ * tiles; the results differ from the tiles' only in the order of the f32 additions.
  */
 int fs2moe_dense_swiglu(const void* x, const void* w_gate, const void* w_up, const void* w_down,
                         int32_t T, int32_t D, int32_t F, int32_t act_dtype, void* h, void* y,
