@@ -81,6 +81,28 @@ def test_ragged_shapes_and_single_tokens(gpu_device, shape):
     assert_output_close(out, ref.out, "bf16")
 
 
+@pytest.mark.parametrize("tokens", [1, 2, 4, 5, 8, 13, 16, 17])
+@pytest.mark.parametrize("mode", ["reference", "softmax"])
+def test_decode_steps_with_a_shared_expert(gpu_device, tokens, mode):
+    """The token counts at which routed and shared experts stream their weights (1-4 rows on the
+    vector ALUs, 5-16 on the matrix pipe; 17: the GEMM tiles), in the reference's routing mode (rows
+    copied and scaled by dispatch) and in softmax mode (rows read through the permutation, dispatch
+    inside the router's second kernel): against the oracle, and single call against stages."""
+    _say("decode step", tokens, mode)
+    rm = W.RoutingMode("sigmoid", False, "input") if mode == "reference" else W.RoutingMode("softmax", True, "output")
+    spec = W.small_spec(tokens=tokens, model_dim=1024, num_experts=16, top_k=2, inner_dim=320, dtype="bf16",
+                        shared=True, zipf_s=1.1, mode=rm, seed=50 + tokens)
+    wl = W.make_workload_from_spec(spec)
+    _, idx, _ = oracle_routing(wl)
+    ref = oracle_forward(wl, idx, 16, dtype=torch.float64)
+    m, x, out, *_ = _run(wl, gpu_device)
+    assert_output_close(out, ref.out, "bf16")
+    with torch.no_grad():
+        single = m(x)  # (out came from the stages)
+    torch.cuda.synchronize()
+    assert torch.equal(single, out)
+
+
 def test_empty_input(gpu_device):
     wl = W.make_workload_from_spec(W.small_spec(tokens=4, dtype="bf16"))
     m = build_module(wl, gpu_device)
