@@ -232,6 +232,55 @@ __global__ __launch_bounds__(kDispTok) void dispatch_small_kernel(
                        s_wave_tot, threadIdx.x, kDispTok);
 }
 
+// All of dispatch for at most 256 tokens WITH the row copy, in one launch: every block works out the
+// bookkeeping for itself in LDS (it is a few microseconds of work, and a decode step spends more on
+// starting three kernels), block 0 writes it to memory, and then the blocks do what
+// dispatch_permute_kernel's do: blocks [0, pair_blocks) copy (and scale) a pair's row per wave,
+// block pair_blocks + e zero-fills the padding rows of expert e.  Same arithmetic, same results.
+template <typename TA>
+__global__ __launch_bounds__(kDispTok) void dispatch_small_copy_kernel(
+    const int32_t* __restrict__ topk_idx, const float* __restrict__ topk_w,
+    const TA* __restrict__ x, int T, int K, int E, int D, int tile_m, int scale_input,
+    int64_t max_rows, unsigned pair_blocks, int32_t* __restrict__ counts,
+    int32_t* __restrict__ offsets, int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm,
+    TA* __restrict__ xe) {
+  extern __shared__ uint32_t s_mem[];
+  __shared__ int32_t s_wave_tot[4];
+  dispatch_small_block(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm, s_mem,
+                       s_wave_tot, threadIdx.x, kDispTok, blockIdx.x == 0);
+  const uint32_t* s_bits = s_mem;
+  const uint32_t* s_pref = s_mem + E * kDispWords;
+  const int32_t* s_off = reinterpret_cast<const int32_t*>(s_pref + E * kDispWords);
+  const int lane = lane_id();
+  const int chunks = D * (int)sizeof(TA) / 16;
+  if (blockIdx.x >= pair_blocks) {
+    const int idx = blockIdx.x - pair_blocks;  // < E
+    const int i = idx * kDispWords + kDispWords - 1;
+    const int cnt = (int)(s_pref[i] + __popc(s_bits[i]));
+    const int64_t lo = (int64_t)s_off[idx] + cnt, hi = s_off[idx + 1];
+    const int64_t n = (hi - lo) * chunks;
+    u32x4* dst = reinterpret_cast<u32x4*>(xe + lo * D);
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int64_t c = threadIdx.x; c < n; c += kDispTok) dst[c] = z;
+    return;
+  }
+  const int64_t p = (int64_t)blockIdx.x * 4 + threadIdx.x / kWave;
+  if (p >= (int64_t)T * K) return;
+  const int t = (int)(p / K);
+  const int e = topk_idx[p];
+  if (e < 0 || e >= E) return;
+  const int w = e * kDispWords + (t >> 5);
+  const int row = s_off[e] + (int)(s_pref[w] + __popc(s_bits[w] & ((1u << (t & 31)) - 1u)));
+  const u32x4* src = reinterpret_cast<const u32x4*>(x + (size_t)t * D);
+  u32x4* dst = reinterpret_cast<u32x4*>(xe + (size_t)row * D);
+  if (scale_input) {
+    const float wt = topk_w[p];
+    for (int c = lane; c < chunks; c += kWave) dst[c] = scale_chunk<TA>(src[c], wt);
+  } else {
+    for (int c = lane; c < chunks; c += kWave) dst[c] = src[c];
+  }
+}
+
 }  // namespace fs2moe
 
 using namespace fs2moe;
@@ -282,6 +331,21 @@ extern "C" int fs2moe_dispatch(const int32_t* topk_idx, const float* topk_w, con
                        dispatch_small_lds_words(E) * sizeof(uint32_t), s, topk_idx, T, K, E,
                        tile_m, max_rows, counts, offsets, perm, inv_perm);
     return check_launch("dispatch_small");
+  }
+  if (nb == 1) {
+    // (xe is given: the copying form of the same)
+    const unsigned pair_blocks = (unsigned)(((int64_t)T * K + 3) / 4);
+    const dim3 grid(pair_blocks + (unsigned)E), block(kDispTok);
+    const size_t lds = dispatch_small_lds_words(E) * sizeof(uint32_t);
+    if (act_dtype == FS2MOE_F32)
+      hipLaunchKernelGGL(dispatch_small_copy_kernel<float>, grid, block, lds, s, topk_idx, topk_w,
+                         static_cast<const float*>(x), T, K, E, D, tile_m, scale_input, max_rows,
+                         pair_blocks, counts, offsets, perm, inv_perm, static_cast<float*>(xe));
+    else
+      hipLaunchKernelGGL(dispatch_small_copy_kernel<uint16_t>, grid, block, lds, s, topk_idx, topk_w,
+                         static_cast<const uint16_t*>(x), T, K, E, D, tile_m, scale_input, max_rows,
+                         pair_blocks, counts, offsets, perm, inv_perm, static_cast<uint16_t*>(xe));
+    return check_launch("dispatch_small_copy");
   }
   if (nb > 0) {
     hipLaunchKernelGGL(dispatch_count_kernel, dim3(nb), dim3(kDispTok),

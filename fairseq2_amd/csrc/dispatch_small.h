@@ -16,13 +16,14 @@ __host__ __device__ inline size_t dispatch_small_lds_words(int E) {
   return (size_t)E * kDispWords * 2 + E + 1;
 }
 
+// write: the results go to memory (else they are only left in LDS: s_bits, s_pref, s_off at s_mem).
 // Called by every thread of a block of `nthreads` >= 256 threads (a multiple of 64); threads 0..255
 // are the tokens' threads, the others only help with the loops over LDS and pass the barriers.
 // topk_idx may have been written by this block before a barrier.
 __device__ __forceinline__ void dispatch_small_block(
     const int32_t* topk_idx, int T, int K, int E, int tile_m, int64_t max_rows, int32_t* counts,
     int32_t* offsets, int32_t* perm, int32_t* inv_perm, uint32_t* s_mem, int32_t* s_wave_tot,
-    int tid, int nthreads) {
+    int tid, int nthreads, bool write = true) {
   uint32_t* s_bits = s_mem;                    // [E][kDispWords] membership bitmaps
   uint32_t* s_pref = s_mem + E * kDispWords;   // [E][kDispWords] members in the words below
   int32_t* s_off = reinterpret_cast<int32_t*>(s_pref + E * kDispWords);  // [E + 1]
@@ -62,7 +63,7 @@ __device__ __forceinline__ void dispatch_small_block(
   if (tid < E) {
     const int i = tid * kDispWords + kDispWords - 1;
     cnt = (int)(s_pref[i] + __popc(s_bits[i]));
-    counts[tid] = cnt;
+    if (write) counts[tid] = cnt;
     padded = (cnt + tile_m - 1) / tile_m * tile_m;
   }
   int incl = padded;
@@ -76,14 +77,16 @@ __device__ __forceinline__ void dispatch_small_block(
   int base = 0;
   for (int w = 0; w < wave && w < 4; ++w) base += s_wave_tot[w];
   if (tid < E) {
-    offsets[tid] = base + incl - padded;
+    if (write) offsets[tid] = base + incl - padded;
     s_off[tid] = base + incl - padded;
   }
   if (tid == E - 1) {
-    offsets[E] = base + incl;
+    if (write) offsets[E] = base + incl;
     s_off[E] = base + incl;
   }
   __syncthreads();
+  // (write false: the bitmaps, prefixes and offsets stay in LDS for the caller, nothing goes to memory)
+  if (!write) return;
   // pairs
 #pragma unroll
   for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) {
