@@ -28,6 +28,9 @@ MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3, "fp8": 5000.0}  # dense, publ
 
 # HBM bytes per launch of the dominant kernel pair, from `rocprofv3 --pmc FETCH_SIZE` and
 # `--pmc WRITE_SIZE` runs of this script (see profiles/); None until measured for a workload.
+# The commit whose kernels the table below was measured on: a kernel change after it makes the
+# figures stale until the counter runs are repeated (the roofline object carries the stamp).
+MEASURED_TRAFFIC_AT = "6025f48"
 MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     # profiles/bench_<workload>_all_kernels.md, the two launches of fs2moe_grouped_swiglu together
     # (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0 against a 256 MiB copy)
@@ -59,10 +62,13 @@ def parse_args():
     p.add_argument("--training-step", action="store_true",
                    help="also time forward + backward of the module (reported beside the metric, "
                         "not part of it; bf16 / fp32 weights only)")
-    p.add_argument("--vendor-gemm", action="store_true",
-                   help="also time the expert GEMM shapes as three dense products in the vendor's "
-                        "library (torch.matmul -> hipBLASLt): a yardstick for what the matrix pipes "
-                        "sustain on this data, reported beside the metric")
+    p.add_argument("--no-vendor-gemm", action="store_true",
+                   help="skip the yardstick that is otherwise reported beside the metric for bf16 "
+                        "workloads: the expert GEMM shapes as three dense products in the vendor's "
+                        "library (torch.matmul -> hipBLASLt) on normally distributed and on all-zero "
+                        "operands, and this build's expert kernels on all-zero operands (what the "
+                        "matrix pipes sustain depends on the operand data: the part is power-limited)")
+    p.add_argument("--vendor-gemm", action="store_true", help="accepted for compatibility: the yardstick is on by default")
     p.add_argument("--calibration-copy", action="store_true",
                    help="also run a 256 MiB device copy (reference point for rocprofv3 byte counters)")
     return p.parse_args()
@@ -207,16 +213,13 @@ def cpu_baseline(wl, seconds: float) -> dict:
 
 def vendor_gemm(spec, dev) -> dict:
     """The routed rows as ONE group through the vendor's dense bf16 GEMM: (T K, D) x (D, F) twice and
-    (T K, F) x (F, D), on data drawn like the workload's.  No grouping, no skew, no gather, no gate:
-    what the same flops cost in the library AMD ships, on this box, on this kind of data."""
+    (T K, F) x (F, D).  No grouping, no skew, no gather, no gate: what the same flops cost in the
+    library AMD ships, on this box.  Timed twice: on data drawn like the workload's, and on all-zero
+    operands, which toggle no bits in the matrix pipes and so show what the same instruction stream
+    reaches when the clock is not held down by power."""
     import torch
 
     rows, d, f = spec.num_tokens * spec.top_k, spec.model_dim, spec.inner_dim
-    g = torch.Generator(device=dev).manual_seed(1)
-    x = torch.randn(rows, d, device=dev, generator=g).to(torch.bfloat16)
-    h = torch.randn(rows, f, device=dev, generator=g).to(torch.bfloat16)
-    w1 = (0.02 * torch.randn(d, f, device=dev, generator=g)).to(torch.bfloat16)
-    w2 = (0.02 * torch.randn(f, d, device=dev, generator=g)).to(torch.bfloat16)
 
     def timed(fn, reps=20):
         for _ in range(10):
@@ -233,16 +236,61 @@ def vendor_gemm(spec, dev) -> dict:
             best = min(best, a.elapsed_time(b) / reps)
         return best
 
-    with torch.no_grad():
-        up_ms = timed(lambda: torch.matmul(x, w1))
-        down_ms = timed(lambda: torch.matmul(h, w2))
-    total = 2 * up_ms + down_ms
     flops = 6.0 * rows * d * f
-    return {
-        "ms": round(total, 4), "gate_or_up_ms": round(up_ms, 4), "down_ms": round(down_ms, 4),
-        "achieved_tflops": round(flops / (total * 1e-3) / 1e12, 1),
-        "what": "torch.matmul (hipBLASLt) on the routed rows as one dense group: gate, up and down products",
-    }
+    out = {"what": "torch.matmul (hipBLASLt) on the routed rows as one dense group: gate, up and down products"}
+    for name in ("normal", "zeros"):
+        if name == "normal":
+            g = torch.Generator(device=dev).manual_seed(1)
+            x = torch.randn(rows, d, device=dev, generator=g).to(torch.bfloat16)
+            h = torch.randn(rows, f, device=dev, generator=g).to(torch.bfloat16)
+            w1 = (0.02 * torch.randn(d, f, device=dev, generator=g)).to(torch.bfloat16)
+            w2 = (0.02 * torch.randn(f, d, device=dev, generator=g)).to(torch.bfloat16)
+        else:
+            x, h = torch.zeros(rows, d, device=dev, dtype=torch.bfloat16), torch.zeros(rows, f, device=dev, dtype=torch.bfloat16)
+            w1, w2 = torch.zeros(d, f, device=dev, dtype=torch.bfloat16), torch.zeros(f, d, device=dev, dtype=torch.bfloat16)
+        with torch.no_grad():
+            up_ms = timed(lambda: torch.matmul(x, w1))
+            down_ms = timed(lambda: torch.matmul(h, w2))
+        total = 2 * up_ms + down_ms
+        ent = {"ms": round(total, 4), "gate_or_up_ms": round(up_ms, 4), "down_ms": round(down_ms, 4),
+               "achieved_tflops": round(flops / (total * 1e-3) / 1e12, 1)}
+        if name == "normal":
+            out.update(ent)
+        else:
+            out["zero_operands"] = ent
+        del x, h, w1, w2
+    return out
+
+
+def experts_on_zero_operands(module, x2, reps: int) -> dict:
+    """This build's expert kernels on the workload's routing with every operand zero (weights and
+    rows): same launches, same tiles, same memory traffic, no bits toggling in the matrix pipes.
+    Zeroes the module's expert weights, so it runs after everything else that uses the module."""
+    import torch
+
+    from fairseq2_amd import _abi
+    from fairseq2_amd.moe import _SCORE_FNS
+
+    ex = module.experts
+    if not (module.scale_on != "input" and hasattr(ex, "fuses_gather") and ex.fuses_gather(x2.dtype)):
+        return {}
+    idx, w, _ = _abi.router_topk(x2, module.router, module.router_bias, module.top_k,
+                                 _SCORE_FNS[module.score_fn], module.renormalize)
+    disp = _abi.dispatch(idx, w, x2, ex.num_local_experts, module.tile_m, False, gather=False)
+    for p in ex.parameters():
+        p.zero_()
+    zx = torch.zeros_like(x2)
+    run = lambda: ex.forward_rows(zx, disp.counts, disp.offsets, row_map=disp.perm)  # noqa: E731
+    for _ in range(10):
+        run()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        run()
+    b.record()
+    torch.cuda.synchronize()
+    return {"ms": round(a.elapsed_time(b) / reps, 4)}
 
 
 def training_step(module, x3, steps: int) -> dict:
@@ -331,6 +379,12 @@ def main() -> int:
             weight, bias, eps, normalized_shape = torch.ones(spec.model_dim, dtype=dt, device=dev), None, 1e-5, (spec.model_dim,)
 
         fused_step = lambda: module(x3, residual=x3, norm=_Norm)  # noqa: E731
+        # settled like the step above: its first calls size buffers the plain step never asked for
+        t_settle = time.perf_counter()
+        while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+            for _ in range(8):
+                fused_step()
+            torch.cuda.synchronize()
         for _ in range(args.warmup):
             fused_step()
         torch.cuda.synchronize()
@@ -400,7 +454,8 @@ def main() -> int:
         roofline = {
             "kernel": kernel, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "launch_ms": round(exp_ms, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "traffic_measured_at": MEASURED_TRAFFIC_AT,
+            "launch_ms": round(exp_ms, 4),
             "bytes_per_launch": work["experts"]["bytes"], "active_experts": active,
         }
     else:
@@ -408,7 +463,8 @@ def main() -> int:
         roofline = {
             "kernel": kernel, "bound": "mfma", "achieved": round(achieved, 2), "peak": peak_tf,
             "unit": "TFLOP/s", "frac": round(achieved / peak_tf, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "launch_ms": round(exp_ms, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "traffic_measured_at": MEASURED_TRAFFIC_AT,
+            "launch_ms": round(exp_ms, 4),
             "flops_per_launch": work["experts"]["flops"],
         }
 
@@ -448,10 +504,18 @@ def main() -> int:
             "what": "x + layer(rms_norm(x)) in one call: norm in the router kernel, residual in combine",
         },
     }
-    if args.vendor_gemm and spec.dtype == "bf16":
-        result["vendor_gemm"] = vendor_gemm(spec, dev)
     if args.training_step and spec.weight_dtype != "fp8":
         result["training_step"] = training_step(module, x3, max(3, args.steps // 10))
+    if not args.no_vendor_gemm and spec.dtype == "bf16" and not experts_hbm_bound:
+        result["vendor_gemm"] = vendor_gemm(spec, dev)
+        if spec.weight_dtype == "bf16":
+            with torch.no_grad():
+                z = experts_on_zero_operands(module, x2, args.stage_reps)
+            if z:
+                z["achieved_tflops"] = round(work["experts"]["flops"] / (z["ms"] * 1e-3) / 1e12, 1)
+                z["what"] = ("this build's two expert kernels, same routing, every operand zero: the same "
+                             "instruction stream and memory traffic without the operands' switching power")
+                result["experts_zero_operands"] = z
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(wl, args.cpu_seconds)
     print(json.dumps(result), flush=True)

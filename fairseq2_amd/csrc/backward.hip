@@ -424,14 +424,21 @@ __global__ __launch_bounds__(256) void pair_dot_kernel(const T* __restrict__ a,
                                                        const T* __restrict__ a2,
                                                        const int32_t* __restrict__ a_rows,
                                                        const T* __restrict__ b, int pairs, int K,
-                                                       int D, float* __restrict__ out) {
+                                                       int D, int vec_ok, float* __restrict__ out) {
   const int p = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (p >= pairs) return;
   const int lane = threadIdx.x & 63;
-  const size_t ar = (size_t)a_rows[p] * D, br = (size_t)(p / K) * D;
+  // A pair whose expert id was out of range has no row (dispatch wrote -1 for it, and combine
+  // skips it): its weight contributed nothing, so its gradient is zero.  Uniform over the wave.
+  const int row = a_rows[p];
+  if (row < 0) {
+    if (lane == 0) out[p] = 0.f;
+    return;
+  }
+  const size_t ar = (size_t)row * D, br = (size_t)(p / K) * D;
   float s = 0.f;
   constexpr int VEC = 16 / sizeof(T);
-  if (D % VEC == 0) {
+  if (vec_ok) {
     // 16 bytes per lane and load
     for (int d = lane * VEC; d < D; d += 64 * VEC) {
       const u32x4 av = *reinterpret_cast<const u32x4*>(a + ar + d);
@@ -660,8 +667,10 @@ __global__ __launch_bounds__(256) void router_backward_kernel(
   }
   if (score_fn == FS2MOE_SCORE_SIGMOID && renormalize) {
     for (int k = 0; k < K; ++k) {
-      const float lk = l[topk_idx[(size_t)t * K + k]];
-      ssum += 1.0f / (1.0f + __expf(-lk));
+      // an id outside [0, E) selects nothing (the forward stages drop such a pair)
+      const int id = topk_idx[(size_t)t * K + k];
+      if (id < 0 || id >= E) continue;
+      ssum += 1.0f / (1.0f + __expf(-l[id]));
     }
   }
   for (int e = lane; e < E; e += 64) {
@@ -829,14 +838,17 @@ extern "C" int fs2moe_pair_dot(const void* a, const void* a2, const int32_t* a_r
   if (pairs == 0) return FS2MOE_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const unsigned blocks = (unsigned)((pairs + 3) / 4);
+  // 16-byte loads need rows that start on 16 bytes: D a multiple of the vector and aligned bases
+  const int vec = 16 / elem_size(dtype);
+  const int vec_ok = D % vec == 0 && aligned16(a) && aligned16(b) && (a2 == nullptr || aligned16(a2));
   if (dtype == FS2MOE_BF16)
     hipLaunchKernelGGL(pair_dot_kernel<uint16_t>, dim3(blocks), dim3(256), 0, st,
                        static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(a2), a_rows,
-                       static_cast<const uint16_t*>(b), (int)pairs, K, D, out);
+                       static_cast<const uint16_t*>(b), (int)pairs, K, D, vec_ok, out);
   else
     hipLaunchKernelGGL(pair_dot_kernel<float>, dim3(blocks), dim3(256), 0, st,
                        static_cast<const float*>(a), static_cast<const float*>(a2), a_rows,
-                       static_cast<const float*>(b), (int)pairs, K, D, out);
+                       static_cast<const float*>(b), (int)pairs, K, D, vec_ok, out);
   return check_launch("pair_dot");
 }
 

@@ -395,7 +395,7 @@ __global__ __launch_bounds__(gemv16::THREADS, DUAL ? 2 : 4) void glu_gemv16_bf16
       if (half > 1) __syncthreads();
     }
     // ---- wave 0: row m = l % 16, channels 8 (4 q + i) + c ---------------------------------------------
-    if (wave == 0 && r0 + c16 < cnt) {
+    if (wave == 0 && row_ok && r0 + c16 < cnt) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int n = blockIdx.x * COLS + (4 * g + i) * 8;
