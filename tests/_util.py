@@ -21,11 +21,13 @@ TORCH_DTYPE = {"fp32": torch.float32, "bf16": torch.bfloat16}
 #   standard deviation sigma ~ 2^-9 * rms(ref) * c, c between 1 and 2 with the SiLU gate's slope
 #   (0.37 % of rms(ref) in the CPU emulation of the rounding points at K = 16 with scaled inputs,
 #   tests/test_oracle_pins.py).  The largest of N such errors is about sqrt(2 ln N) sigma: 5.3 sigma
-#   = 2 % of rms(ref) for the 5.6e5 elements of a 1100 x 512 output, so atol = 2 % sits AT the expected
-#   maximum (a seeded case did land at 1.03 of it); atol = 4e-2 * rms is 10 sigma.  The overall
-#   statement, RMS_TOL = 1e-2, is the sharp one: 2.7 sigma-units above the emulation's 0.37 %.
+#   = 2 % of rms(ref) for the 5.6e5 elements of a 1100 x 512 output: with that many elements, K >= 8
+#   and the rows scaled on the way in (a fourth rounding per term), atol = 2 % sits AT the expected
+#   maximum (a seeded case did land at 1.03 of it).  Such cases, and only they, pass atol_scale = 2
+#   (4e-2 * rms, 10 sigma); everything else is held to 2e-2.  The overall statement, RMS_TOL = 1e-2,
+#   is the sharp one everywhere: 2.7 sigma-units above the emulation's 0.37 %.
 # fp32: rtol 1e-4, atol 1e-4 * rms, RMS_TOL 2e-5 (f32 MFMA accumulation order differs from the CPU's).
-TOL = {"bf16": (2e-2, 4e-2), "fp32": (1e-4, 1e-4)}
+TOL = {"bf16": (2e-2, 2e-2), "fp32": (1e-4, 1e-4)}
 RMS_TOL = {"bf16": 1e-2, "fp32": 2e-5}
 
 
@@ -49,10 +51,12 @@ def oracle_forward(wl: W.Workload, idx, tile_m: int, tokens=None, dtype=torch.fl
     )
 
 
-def assert_output_close(got: torch.Tensor, ref: torch.Tensor, dtype: str, what: str = "output"):
+def assert_output_close(got: torch.Tensor, ref: torch.Tensor, dtype: str, what: str = "output",
+                        atol_scale: float = 1.0):
     got = got.detach().double().cpu().reshape(ref.shape)
     ref = ref.double()
     rtol, atol_rel = TOL[dtype]
+    atol_rel *= atol_scale
     rms = float(ref.pow(2).mean().sqrt())
     atol = atol_rel * rms
     err = (got - ref).abs()

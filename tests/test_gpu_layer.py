@@ -725,7 +725,10 @@ def test_reference_arithmetic_in_bf16(gpu_device):
     same = (torch.sort(ref_idx, dim=1).values == torch.sort(gi.cpu().long(), dim=1).values).all(dim=1)
     assert float(same.float().mean()) > 0.9
     got = out.reshape(-1, 128).cpu()[same]
-    assert_output_close(got, dense_bf16.reshape(-1, 128)[same].double(), "bf16", "vs the reference in bf16")
+    # both sides carry bf16 rounding here, and the reference's side more of it (scores rounded to
+    # bf16 scale whole rows, scatter_add_ rounds after every addition): twice the element-wise room
+    assert_output_close(got, dense_bf16.reshape(-1, 128)[same].double(), "bf16", "vs the reference in bf16",
+                        atol_scale=2.0)
 
 
 def test_layer_arguments_are_validated_before_the_gpu_reads_them(gpu_device):

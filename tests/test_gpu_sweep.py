@@ -149,7 +149,9 @@ def test_seeded_sweep(gpu_device, seed):
         ref = oracle_forward(wl, idx, c["tile_m"], dtype=torch.float64)
         want = ref.out if res_c is None else ref.out + res_c.double()
         assert_routing_equal(gi, disp, ref.routing, f"case {it}")
-        assert_output_close(single, want, c["dtype"], f"case {it}")
+        # many terms, each rounded a fourth time on the way in: see tests/_util.py
+        many_roundings = c["k"] >= 8 and c["mode"].scale_on == "input"
+        assert_output_close(single, want, c["dtype"], f"case {it}", atol_scale=2.0 if many_roundings else 1.0)
         if random.Random(1000 * seed + it).random() < 0.35:
             _check_norm_in_front(m, c, dt, res, gpu_device, it)
     print(f"sweep seed={seed}: {len(cases)} cases, {near_ties} with near-ties resolved through the host mirror", flush=True)
