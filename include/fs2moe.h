@@ -271,6 +271,8 @@ int fs2moe_forward_norm(const void* x, const void* norm_weight, float norm_eps,
  *   rejected with FS2MOE_ERR_ARG (decode-sized batches fit; prefill-sized ones do not).
  *   All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
  *   streams or threads) race and must be serialised by the caller.
+ *   The first call on a device looks up the array's address and sets kernel attributes (host-side
+ *   work, no allocation): make it once outside any stream capture before capturing later calls.
  */
 int64_t fs2moe_forward_static_capacity(void);
 int fs2moe_forward_static(const void* x, const void* residual, const void* router,

@@ -93,6 +93,49 @@ def test_static_scratch_entry_point_equals_forward(gpu_device, dtype, fp8, mode,
 
 
 @pytest.mark.gpu
+def test_static_scratch_call_allocates_nothing_and_runs_up_to_its_capacity(gpu_device):
+    """After one call on the device (which looks the array's address up and sets function
+    attributes), a call changes neither the device's free memory nor torch's allocation count.
+    Also the largest token count whose intermediates still fit the array, against fs2moe_forward."""
+    print("forward_static at capacity", flush=True)
+    lib = _abi.load()
+    d, e, k, f, tile_m = 256, 16, 2, 128, 16
+    cap = lib.fs2moe_forward_static_capacity()
+    need = lambda t: lib.fs2moe_forward_workspace_bytes(t, d, e, k, f, 0, tile_m, _abi.BF16)  # noqa: E731
+    lo, hi = 1, 1 << 20
+    assert need(lo) <= cap < need(hi)
+    while hi - lo > 1:  # need() grows with the token count
+        mid = (lo + hi) // 2
+        lo, hi = (mid, hi) if need(mid) <= cap else (lo, mid)
+    t_max = lo
+    assert need(t_max) <= cap < need(t_max + 1)
+    spec = W.small_spec(tokens=t_max, model_dim=d, num_experts=e, top_k=k, inner_dim=f, dtype="bf16", zipf_s=1.1,
+                        mode=W.RoutingMode("softmax", True, "output"), seed=62)
+    wl = W.make_workload_from_spec(spec)
+    m = build_module(wl, gpu_device, tile_m)
+    x = wl.x.to(torch.bfloat16).to(gpu_device).reshape(-1, d).contiguous()
+    want, got = _both_ways(lib, m, wl, x, None, False, tile_m)
+    assert torch.equal(got, want), f"T={t_max}, {need(t_max)} of {cap} bytes"
+    # one token more is refused
+    w, s, sh, _ = _layer_args(m, wl, False)
+    out = torch.empty((t_max + 1, d), dtype=torch.bfloat16, device=gpu_device)
+    xx = torch.zeros((t_max + 1, d), dtype=torch.bfloat16, device=gpu_device)
+    stream = torch.cuda.current_stream().cuda_stream
+    args = lambda rows, dst: (  # noqa: E731
+        _ptr(rows), None, _ptr(m.router.detach()), _ptr(m.router_bias), *map(_ptr, w), *map(_ptr, s), *map(_ptr, sh),
+        rows.shape[0], d, e, k, f, 0, tile_m, _abi.BF16, _abi.BF16, _SCORE_FNS["softmax"], 1, 0, _ptr(dst), stream)
+    assert lib.fs2moe_forward_static(*args(xx, out)) == -1
+    # a warmed call allocates nothing
+    got2 = torch.empty_like(x)
+    torch.cuda.synchronize()
+    free0, alloc0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
+    assert lib.fs2moe_forward_static(*args(x, got2)) == 0, lib.fs2moe_last_error()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_allocated() == alloc0
+    assert torch.equal(got2, want)
+
+
+@pytest.mark.gpu
 def test_static_scratch_rejects_what_does_not_fit(gpu_device):
     print("forward_static too large", flush=True)
     lib = _abi.load()
