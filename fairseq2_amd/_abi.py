@@ -15,7 +15,7 @@ from torch import Tensor
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfs2moe.so")
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
@@ -132,6 +132,11 @@ _PROTOTYPES = {
         c_int32,
         [c_void_p, c_void_p, c_float, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p,
          c_void_p, c_int64, c_void_p],
+    ),
+    "fs2moe_mx_quantize": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p]),
+    "fs2moe_grouped_swiglu_w8a8_supported": (c_int32, [c_int32, c_int32, c_int64]),
+    "fs2moe_grouped_swiglu_w8a8": (
+        c_int32, [c_void_p] * 11 + [c_int32] * 3 + [c_int64] + [c_void_p] * 4,
     ),
     "fs2moe_forward_norm": (
         c_int32,
@@ -458,6 +463,69 @@ def grouped_swiglu(
 def keeps_products(model_dim: int, inner_dim: int, rows: int, act_dtype: torch.dtype) -> bool:
     """Whether :func:`grouped_swiglu_keep` exists for these sizes and this type."""
     return bool(load().fs2moe_grouped_swiglu_keeps(model_dim, inner_dim, rows, dtype_code(act_dtype)))
+
+
+def mx_quantize(x: Tensor) -> tuple[Tensor, Tensor]:
+    """bf16 rows ``(rows, D)`` -> e4m3 codes ``(rows, D)`` (as uint8) and one exponent byte per row
+    and 32 features ``(rows, D / 32)`` (``fs2moe_mx_quantize``)."""
+    lib = load()
+    if x.dim() != 2 or x.dtype != torch.bfloat16 or x.shape[1] % 32:
+        raise ValueError("mx_quantize takes (rows, D) bf16 with D a multiple of 32")
+    rows, d = x.shape
+    codes = torch.empty((rows, d), dtype=torch.uint8, device=x.device)
+    scales = torch.empty((rows, d // 32), dtype=torch.uint8, device=x.device)
+    rc = lib.fs2moe_mx_quantize(_ptr(x), rows, d, _ptr(codes), _ptr(scales), _stream())
+    _check(rc, "fs2moe_mx_quantize")
+    return codes, scales
+
+
+def w8a8_supported(model_dim: int, inner_dim: int, rows: int) -> bool:
+    return bool(load().fs2moe_grouped_swiglu_w8a8_supported(model_dim, inner_dim, rows))
+
+
+def grouped_swiglu_w8a8(
+    xq: Tensor,
+    xs: Tensor,
+    counts: Tensor,
+    offsets: Tensor,
+    w_gate: Tensor,
+    w_up: Tensor,
+    w_down: Tensor,
+    scales: tuple[Tensor, Tensor, Tensor],
+    num_experts: int,
+    row_map: Tensor | None = None,
+) -> tuple[Tensor, Tensor, Tensor]:
+    """The grouped SwiGLU network on the fp8 matrix pipe (``fs2moe_grouped_swiglu_w8a8``): block-scaled
+    e4m3 rows (:func:`mx_quantize`) against tiled e4m3 weights with channel scales.  Returns
+    ``(ye, hq, hs)``: bf16 output rows and the quantised gated product."""
+    lib = load()
+    rows, d = xq.shape
+    dev = xq.device
+    _same("xq", xq, (rows, d), torch.uint8, dev)
+    _same("xs", xs, (rows, d // 32), torch.uint8, dev)
+    if row_map is not None:
+        if row_map.dtype != torch.int32 or row_map.dim() != 1:
+            raise ValueError("row_map must be a 1-d int32 tensor")
+        rows = row_map.shape[0]
+    _check_groups(counts, offsets, num_experts, dev)
+    f = w_gate.shape[1] * 16
+    if w_gate.shape != (num_experts, f // 16, d // 64, 16, 64) or w_up.shape != w_gate.shape:
+        raise ValueError("fp8 gate/up codes must be tiled (E, F/16, D/64, 16, 64)")
+    if w_down.shape != (num_experts, d // 16, f // 64, 16, 64):
+        raise ValueError("fp8 down codes must be tiled (E, D/16, F/64, 16, 64)")
+    want = [(num_experts, f), (num_experts, f), (num_experts, d)]
+    if [tuple(s.shape) for s in scales] != want or any(s.dtype != torch.float32 for s in scales):
+        raise ValueError("fp8 scales must be f32 (E, F), (E, F), (E, D)")
+    hq = torch.empty((rows, f), dtype=torch.uint8, device=dev)
+    hs = torch.empty((rows, f // 32), dtype=torch.uint8, device=dev)
+    ye = torch.empty((rows, d), dtype=torch.bfloat16, device=dev)
+    rc = lib.fs2moe_grouped_swiglu_w8a8(
+        _ptr(xq), _ptr(xs), _ptr(row_map), _ptr(counts), _ptr(offsets), _ptr(w_gate), _ptr(w_up),
+        _ptr(w_down), _ptr(scales[0]), _ptr(scales[1]), _ptr(scales[2]), num_experts, d, f, rows,
+        _ptr(hq), _ptr(hs), _ptr(ye), _stream(),
+    )
+    _check(rc, "fs2moe_grouped_swiglu_w8a8")
+    return ye, hq, hs
 
 
 def grouped_swiglu_keep(

@@ -17,7 +17,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfs2moe.so")
 
-SOURCES = ["abi.hip", "router.hip", "dispatch.hip", "experts.hip", "combine.hip", "backward.hip"]
+SOURCES = ["abi.hip", "router.hip", "dispatch.hip", "experts.hip", "combine.hip", "backward.hip", "mx.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

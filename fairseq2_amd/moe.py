@@ -104,10 +104,27 @@ class GroupedExpertNetwork(ExpertNetwork):
         # Any module, as in the reference (experts.py:84-87).  The fused kernels implement the SiLU
         # gate; another activation runs between plain grouped GEMMs of the same library.
         self.activation = activation if activation is not None else nn.SiLU()
+        # Opt-in (no counterpart in the reference): "mxfp8" rounds the inputs of the expert products
+        # to block-scaled e4m3 so that, with e4m3 weights, they run on the fp8 matrix pipe (W8A8).
+        self.act_quant: str | None = None
 
     @property
     def has_fused_gate(self) -> bool:
         return isinstance(self.activation, nn.SiLU)
+
+    # e4m3 weights go to the GEMM kernels from this many rows per expert on (mean over all experts,
+    # the library's own rule for its bf16-pipe path); below that the experts are a weight stream,
+    # which activations of one byte would not make faster.
+    _W8A8_MIN_ROWS_PER_EXPERT = 32
+
+    def runs_w8a8(self, act_dtype: torch.dtype, rows: int) -> bool:
+        """Whether :meth:`forward_rows` on ``rows`` rows takes the fp8 matrix pipe."""
+        return (
+            self.act_quant == "mxfp8" and self.has_fp8_weights and self.has_fused_gate
+            and act_dtype == torch.bfloat16
+            and rows // self.num_local_experts >= self._W8A8_MIN_ROWS_PER_EXPERT
+            and _abi.w8a8_supported(self.model_dim, self.inner_dim, rows)
+        )
 
     # ---- fp8 (e4m3) weights: derived, non-persistent buffers next to the Parameters ----------------
     # Stored as integers (codes as uint8, scales as the int32 bit patterns of their f32 values) so
@@ -236,6 +253,17 @@ class GroupedExpertNetwork(ExpertNetwork):
             u = _abi.grouped_gemm(xe, self.inner_proj.detach(), _abi.W_IN_OUT, **grp)
             h = (self.activation(g.float()) * u.float()).to(xe.dtype)
             return _abi.grouped_gemm(h.contiguous(), self.output_proj.detach(), _abi.W_IN_OUT, **grp)
+        rows = xe.shape[0] if row_map is None else row_map.shape[0]
+        if self.runs_w8a8(xe.dtype, rows):
+            # the rows (the token matrix when they are read through a map) to block-scaled e4m3,
+            # then both products on the fp8 matrix pipe
+            xq, xs = _abi.mx_quantize(xe)
+            ye, _, _ = _abi.grouped_swiglu_w8a8(
+                xq, xs, counts, offsets, self.gate_q, self.inner_q, self.output_q,
+                (self.gate_scale, self.inner_scale, self.output_scale), self.num_local_experts,
+                row_map=row_map,
+            )
+            return ye
         if self.has_fp8_weights:
             ye, _ = _abi.grouped_swiglu(
                 xe, counts, offsets, self.gate_q, self.inner_q, self.output_q,
@@ -396,8 +424,11 @@ class MoE(FeedForwardNetwork):
         scale_on: str = "input",
         router_bias: bool = False,
         tile_m: int = 16,
+        act_quant: str | None = None,
     ) -> None:
         super().__init__()
+        if act_quant not in (None, "mxfp8"):
+            raise ValueError(f"act_quant must be None or 'mxfp8', got {act_quant!r}")
         if score_fn not in _SCORE_FNS:
             raise ValueError(f"score_fn must be 'sigmoid' or 'softmax', got {score_fn!r}")
         if scale_on not in ("input", "output"):
@@ -435,6 +466,8 @@ class MoE(FeedForwardNetwork):
         self.router = Parameter(torch.empty(model_dim, num_experts))
         self.top_k = top_k
         self.experts = GroupedExpertNetwork(num_experts, model_dim, inner_dim, activation=moe_activation)
+        # keyword-only extension, off by default: see GroupedExpertNetwork.act_quant
+        self.experts.act_quant = act_quant
 
         # Kept for interface parity; tensor-parallel reduction is outside the single-GPU path.
         self.tp_gang = None
@@ -491,7 +524,9 @@ class MoE(FeedForwardNetwork):
         if x.shape[0] == 0:
             return torch.empty_like(seqs)
         ex, se = self.experts, self.shared_expert
-        if (type(ex) is GroupedExpertNetwork and ex.has_fused_gate
+        w8a8 = type(ex) is GroupedExpertNetwork and ex.runs_w8a8(
+            x.dtype, x.shape[0] * self.top_k + ex.num_local_experts * (self.tile_m - 1))
+        if (type(ex) is GroupedExpertNetwork and ex.has_fused_gate and not w8a8
                 and (se is None or type(se) is GLUFeedForwardNetwork)):
             return self._single_call(x, res, norm_args).view(seqs.shape)
         if wants_grad:

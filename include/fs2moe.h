@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FS2MOE_ABI_VERSION 12
+#define FS2MOE_ABI_VERSION 13
 
 /* element types */
 #define FS2MOE_F32 0
@@ -260,6 +260,34 @@ int fs2moe_forward_norm(const void* x, const void* norm_weight, float norm_eps,
                         int32_t tile_m, int32_t act_dtype, int32_t w_dtype, int32_t score_fn,
                         int32_t renormalize, int32_t scale_input, void* workspace,
                         int64_t workspace_bytes, void* out, void* stream);
+
+/*
+ * W8A8: the experts on the fp8 matrix pipe, an opt-in of this library with no counterpart in the
+ * reference (its experts run in the parameters' dtype, models/transformer/experts.py:102-112).
+ * Weights are the e4m3 codes and per-output-channel scales of fs2moe_grouped_swiglu (w_dtype
+ * FS2MOE_FP8_E4M3); activations are e4m3 codes with one power-of-two scale per row and block of 32
+ * consecutive features, stored as the exponent byte X + 127:
+ *     X = the smallest integer with max|block| / 2^X <= 448   (-127 for a zero block)
+ *     code = e4m3(value / 2^X), round to nearest even         value ~ code * 2^X
+ *
+ * fs2moe_mx_quantize: x [rows, D] bf16 -> codes [rows, D] (1 byte each) and scales [rows, D / 32];
+ *   D a multiple of 32.
+ * fs2moe_grouped_swiglu_w8a8: the grouped SwiGLU network of fs2moe_grouped_swiglu on such rows.
+ *   xq [T or max_rows, D] codes, xs [.., D / 32] scales, both read through row_map [max_rows] when it
+ *   is given (the gather of moe.py:131 fused into the first product), else expert-major;
+ *   hq [max_rows, F] / hs [max_rows, F / 32]: the gated product, quantised the same way by the first
+ *   kernel's epilogue (from its f32 values) and read by the second; ye [max_rows, D] bf16.
+ *   D and F multiples of 128 (fs2moe_grouped_swiglu_w8a8_supported says whether sizes qualify).
+ */
+int fs2moe_mx_quantize(const void* x, int64_t rows, int32_t D, void* codes, void* scales,
+                       void* stream);
+int fs2moe_grouped_swiglu_w8a8_supported(int32_t D, int32_t F, int64_t max_rows);
+int fs2moe_grouped_swiglu_w8a8(const void* xq, const void* xs, const int32_t* row_map,
+                               const int32_t* counts, const int32_t* offsets, const void* w_gate,
+                               const void* w_up, const void* w_down, const float* s_gate,
+                               const float* s_up, const float* s_down, int32_t E, int32_t D,
+                               int32_t F, int64_t max_rows, void* hq, void* hs, void* ye,
+                               void* stream);
 
 /*
  * The whole layer without a workspace argument, for callers that cannot allocate device memory

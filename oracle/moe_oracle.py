@@ -43,8 +43,11 @@ ties to the lower expert id, NaN ranks above everything (as in torch).
 
 Extensions beyond the reference (defaults reproduce it): a per-expert router
 bias, ``score_fn="softmax"`` with optional renormalisation over the selected
-experts, and ``scale_on="output"`` (weight the expert output instead of the
-expert input).
+experts, ``scale_on="output"`` (weight the expert output instead of the
+expert input), and ``act_quant="mxfp8"``: the inputs of the two expert
+products rounded to block-scaled e4m3 (``mx_quantize``; the cast itself is
+PyTorch's ``float8_e4m3fn`` conversion, pinned against a brute-force nearest
+search over all 256 codes in ``tests/test_oracle_pins.py``).
 """
 
 from __future__ import annotations
@@ -191,6 +194,48 @@ def route(topk_idx: Tensor | np.ndarray, num_experts: int, tile_m: int = 1) -> R
 
 
 # --------------------------------------------------------------------------- a6
+# ------------------------------------------------------------ block-scaled e4m3
+MX_BLOCK = 32
+E4M3_MAX = 448.0
+
+
+def mx_block_exponent(amax: Tensor) -> Tensor:
+    """The shared exponent X of blocks with the given largest magnitudes: the smallest integer with
+    ``amax / 2**X <= 448``, i.e. for ``amax = m 2**e`` with ``m`` in [1, 2): ``e - 8`` when
+    ``m <= 1.75``, else ``e - 7``.  Zero blocks (and magnitudes below the smallest normal float32)
+    get -127; the result is clamped to [-127, 127] (what one byte, X + 127, can say)."""
+    a = amax.detach().to(torch.float32)
+    m, e = torch.frexp(a)  # a = m 2**e with m in [0.5, 1)
+    x = e.to(torch.int32) - 1 - 8 + (m > 0.875).to(torch.int32)
+    x = torch.where(a < 2.0 ** -126, torch.full_like(x, -127), x)
+    return x.clamp(-127, 127)
+
+
+def mx_quantize(x: Tensor) -> tuple[Tensor, Tensor]:
+    """Rows ``(*, D)`` -> e4m3 codes ``(*, D)`` (``torch.float8_e4m3fn``) and exponent bytes
+    ``(*, D / 32)`` (uint8, X + 127): every block of 32 consecutive features is divided by
+    ``2**X`` (exact) and rounded to e4m3, to nearest, ties to even."""
+    d = x.shape[-1]
+    assert d % MX_BLOCK == 0
+    v = x.detach().to(torch.float32).reshape(*x.shape[:-1], d // MX_BLOCK, MX_BLOCK)
+    xexp = mx_block_exponent(v.abs().amax(dim=-1))
+    scaled = torch.ldexp(v, -xexp.unsqueeze(-1))
+    codes = scaled.to(torch.float8_e4m3fn).reshape(x.shape)
+    return codes, (xexp + 127).to(torch.uint8)
+
+
+def mx_dequantize(codes: Tensor, scale_bytes: Tensor, dtype: torch.dtype = torch.float32) -> Tensor:
+    d = codes.shape[-1]
+    v = codes.to(torch.float32).reshape(*codes.shape[:-1], d // MX_BLOCK, MX_BLOCK)
+    x = scale_bytes.to(torch.int32) - 127
+    return torch.ldexp(v, x.unsqueeze(-1)).reshape(codes.shape).to(dtype)
+
+
+def mx_round(x: Tensor) -> Tensor:
+    """``x`` as the fp8 matrix pipe sees it: quantised and de-quantised, in ``x``'s dtype."""
+    return mx_dequantize(*mx_quantize(x), dtype=x.dtype)
+
+
 def glu_expert(u: Tensor, wg: Tensor, wu: Tensor, wd: Tensor) -> Tensor:
     """One expert: ``(SiLU(u @ Wg) * (u @ Wu)) @ Wd`` (``experts.py:107-112``)."""
     return (F.silu(u @ wg) * (u @ wu)) @ wd
@@ -298,14 +343,20 @@ def ref_sparse_forward(
     tile_m: int = 1,
     topk_idx: Tensor | None = None,
     tokens: Tensor | None = None,
+    act_quant: str | None = None,
 ) -> SparseResult:
     """Per-expert evaluation of the layer on only the routed tokens.
+
+    ``act_quant="mxfp8"``: the rows entering the gate/up products and the gated product entering
+    the down projection are rounded to block-scaled e4m3 first (``mx_round``); the router, the
+    shared expert and the combination see the unrounded rows.
 
     ``topk_idx`` may be supplied to evaluate with a given selection.  ``tokens``
     restricts the expert evaluation to a subset of token ids (the output rows of
     all other tokens are left at the base value); routing artefacts always cover
     every token.
     """
+    assert act_quant in (None, "mxfp8")
     dim = seqs.shape[-1]
     x = seqs.reshape(-1, dim)
     t = x.shape[0]
@@ -352,7 +403,14 @@ def ref_sparse_forward(
         if scale_on == "input":
             u = u * row_w[rows, None]
         xe[rows] = u
+        if act_quant == "mxfp8":
+            # the quantiser reads bf16 rows (the dtype this option exists for): rows scaled on the
+            # way in are rounded to bf16 first, as the gathered copy holds them; rows that are
+            # bf16 values already pass through that unchanged
+            u = mx_round(u.to(torch.bfloat16).to(u.dtype))
         he = F.silu(u @ wg[e]) * (u @ wu[e])
+        if act_quant == "mxfp8":
+            he = mx_round(he)
         h[rows] = he
         ye[rows] = he @ wd[e]
 

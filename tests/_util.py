@@ -40,7 +40,7 @@ def oracle_routing(wl: W.Workload):
     return logits, idx, w
 
 
-def oracle_forward(wl: W.Workload, idx, tile_m: int, tokens=None, dtype=torch.float32):
+def oracle_forward(wl: W.Workload, idx, tile_m: int, tokens=None, dtype=torch.float32, act_quant="spec"):
     c = lambda t: None if t is None else t.to(dtype)
     shared = (c(wl.shared_gate), c(wl.shared_up), c(wl.shared_down)) if wl.spec.shared else None
     return O.ref_sparse_forward(
@@ -48,6 +48,7 @@ def oracle_forward(wl: W.Workload, idx, tile_m: int, tokens=None, dtype=torch.fl
         shared=shared, router_bias=c(wl.router_bias),
         score_fn=wl.spec.mode.score_fn, renormalize=wl.spec.mode.renormalize,
         scale_on=wl.spec.mode.scale_on, tile_m=tile_m, topk_idx=idx, tokens=tokens,
+        act_quant=wl.spec.act_quant if act_quant == "spec" else act_quant,
     )
 
 

@@ -485,8 +485,8 @@ def test_bf16_rounding_budget_of_the_device_pipeline():
     bf16 rounding wherever the device rounds, against the f64 oracle, in the configuration with the
     most roundings per output element (every one of 16 experts selected, scaled input rows).  The
     overall error is a few tenths of a percent of the output's rms, well inside RMS_TOL, and every
-    element is inside the element-wise bound with room to spare (the largest errors sit on the largest
-    elements, where the final rounding alone is 2^-9 of the value: they are what rtol is for)."""
+    element is inside the element-wise bound (the largest errors sit on the largest elements, where
+    the final rounding alone is 2^-9 of the value: they are what rtol is for)."""
     import workloads as W
     from tests._util import RMS_TOL, TOL, emulate_device_rounding, oracle_forward, oracle_routing
 
@@ -502,7 +502,109 @@ def test_bf16_rounding_budget_of_the_device_pipeline():
     assert 5e-4 < sigma < 6e-3, sigma  # ~ 2^-9 .. 3 * 2^-9
     assert sigma < 0.6 * RMS_TOL["bf16"]
     rtol, atol_rel = TOL["bf16"]
-    worst = float((err / (atol_rel * rms + rtol * ref.abs())).max())
+    assert atol_rel == 2e-2
+    # this configuration (K >= 8 terms, each rounded a fourth time on the way in) is the one the GPU
+    # tests give twice the element-wise room (atol_scale = 2): with it every element is well inside,
+    worst = float((err / (2 * atol_rel * rms + rtol * ref.abs())).max())
     assert worst < 0.6, worst
-    # with atol = 2e-2 * rms the same elements come close to the bound: no room for the tail
-    assert float((err / (2e-2 * rms + rtol * ref.abs())).max()) > 0.6
+    # while at the default the same elements come close to the bound: no room for the tail of a
+    # larger output
+    assert 0.6 < float((err / (atol_rel * rms + rtol * ref.abs())).max()) < 1.0
+
+
+# ------------------------------------------------------------------ block-scaled e4m3 (act_quant)
+def _e4m3_values():
+    """Every finite e4m3fn value by the format's definition (1 sign, 4 exponent bits with bias 7,
+    3 mantissa bits, no infinities, 0x7f / 0xff are NaN), in pure Python: code -> value."""
+    vals = {}
+    for code in range(256):
+        if code & 0x7F == 0x7F:
+            continue
+        s, e, m = code >> 7, (code >> 3) & 15, code & 7
+        v = (m / 8.0) * 2.0 ** -6 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7)
+        vals[code] = -v if s else v
+    return vals
+
+
+def test_mx_block_exponent_closed_forms():
+    f32 = torch.float32
+    n = torch.arange(-20, 21)
+    top = torch.ldexp(torch.tensor(448.0), n)  # 448 * 2^n fits exactly: X = n
+    assert O.mx_block_exponent(top).tolist() == n.tolist()
+    above = torch.nextafter(top, torch.tensor(float("inf")))  # one ulp more needs the next exponent
+    assert O.mx_block_exponent(above).tolist() == (n + 1).tolist()
+    assert O.mx_block_exponent(torch.tensor([1.0, 1.75, 1.7500001, 2.0, 224.0, 255.9, 256.0], dtype=f32)).tolist() == [
+        -8, -8, -7, -7, -1, 0, 0]
+    assert O.mx_block_exponent(torch.tensor([0.0, 1e-45, 2.0 ** -127], dtype=f32)).tolist() == [-127, -127, -127]
+    assert O.mx_block_exponent(torch.tensor([2.0 ** -126, 2.9e38, 3e38], dtype=f32)).tolist() == [-127, 119, 120]
+    # the defining property on random magnitudes: amax / 2^X <= 448 < amax / 2^(X - 1)
+    g = torch.Generator().manual_seed(5)
+    a = torch.exp(20 * torch.rand(4096, generator=g) - 10).to(f32)
+    x = O.mx_block_exponent(a)
+    assert bool((torch.ldexp(a.double(), -x) <= 448).all())
+    assert bool((torch.ldexp(a.double(), -(x - 1)) > 448).all())
+
+
+def test_mx_quantize_is_the_nearest_code_with_ties_to_even():
+    """Brute force over the table of all codes: the quantised value of every element is the e4m3
+    value nearest to element / 2^X, and on a tie the one with the even code."""
+    vals = _e4m3_values()
+    table = sorted((v, c) for c, v in vals.items() if c < 0x80)  # non-negative half
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(24, 64, generator=g) * torch.exp(3 * torch.randn(24, 1, generator=g))).to(torch.bfloat16)
+    x[0, :32] = 0
+    x[1, :4] = torch.tensor([17.0, 19.0, 448.0, 0.0009765625])  # exact ties below a larger element
+    x[1, 4] = 28.0
+    codes, sb = O.mx_quantize(x)
+    got = codes.view(torch.uint8).reshape(24, 2, 32)
+    for r in range(24):
+        for b in range(2):
+            blk = x[r, 32 * b : 32 * b + 32].double()
+            amax = float(blk.abs().max())
+            xexp = int(sb[r, b]) - 127
+            if amax == 0:
+                assert xexp == -127 and int(got[r, b].sum()) == 0
+                continue
+            assert amax / 2.0 ** xexp <= 448 < amax / 2.0 ** (xexp - 1)
+            for i in range(32):
+                t = abs(float(blk[i])) / 2.0 ** xexp
+                best = min(table, key=lambda vc: (abs(vc[0] - t), vc[1] & 1))
+                want = best[1] | (0x80 if float(blk[i]) < 0 else 0)
+                have = int(got[r, b, i])
+                assert vals[have] == vals[want], (r, b, i, float(blk[i]), have, want)
+    # and the round trip: exact for what e4m3 holds, within 2^-4 of the value (normal range) or
+    # 2^-10 of the block's scale (below it) otherwise
+    back = O.mx_dequantize(codes, sb).double().reshape(24, 2, 32)
+    xs = x.double().reshape(24, 2, 32)
+    scale = torch.ldexp(torch.ones(24, 2, dtype=torch.float64), sb.to(torch.int32) - 127).unsqueeze(-1)
+    err = (back - xs).abs()
+    assert bool((err <= torch.maximum(xs.abs() * 2.0 ** -4, scale * 2.0 ** -10) + 1e-300).all())
+    pow2 = torch.ldexp(torch.ones(1, 32), torch.arange(-3, 5).repeat(4).unsqueeze(0))
+    assert torch.equal(O.mx_round(pow2), pow2)
+
+
+def test_sparse_forward_with_quantised_activations_is_the_layer_on_rounded_inputs():
+    """act_quant="mxfp8" against the composition written out by hand for one expert and one token
+    per row group: round the rows, multiply, gate, round the product, multiply."""
+    g = torch.Generator().manual_seed(3)
+    t, d, f, e = 6, 64, 32, 2
+    x = torch.randn(t, d, generator=g, dtype=torch.float64).to(torch.bfloat16).double()  # bf16 rows
+    router = torch.randn(d, e, generator=g, dtype=torch.float64)
+    gate, up = (0.2 * torch.randn(e * d, f, generator=g, dtype=torch.float64) for _ in range(2))
+    down = 0.2 * torch.randn(e * f, d, generator=g, dtype=torch.float64)
+    res = O.ref_sparse_forward(x, router, gate, up, down, 1, score_fn="softmax", renormalize=True,
+                               scale_on="output", act_quant="mxfp8")
+    plain = O.ref_sparse_forward(x, router, gate, up, down, 1, score_fn="softmax", renormalize=True,
+                                 scale_on="output")
+    assert torch.equal(res.topk_idx, plain.topk_idx), "the router sees the unrounded rows"
+    want = torch.zeros(t, d, dtype=torch.float64)
+    for i in range(t):
+        ex = int(res.topk_idx[i, 0])
+        u = O.mx_round(x[i : i + 1])
+        h = torch.nn.functional.silu(u @ gate.view(e, d, f)[ex]) * (u @ up.view(e, d, f)[ex])
+        want[i] = (O.mx_round(h) @ down.view(e, f, d)[ex])[0]  # weight 1: one expert, renormalised
+    torch.testing.assert_close(res.out, want, rtol=1e-12, atol=1e-12)
+    rel = float((res.out - plain.out).norm() / plain.out.norm())
+    # the format's noise: three mantissa bits leave every element off by up to 2^-4 of its size
+    # (3.6 % rms), at two places of the pipeline, so some 5-6 % of the output's norm
+    assert 2e-2 < rel < 1e-1, rel

@@ -58,6 +58,7 @@ class WorkloadSpec:
     zipf_s: float | None
     shared: bool
     mode: RoutingMode
+    act_quant: str | None = None  # "mxfp8": the experts' inputs in block-scaled e4m3 (W8A8)
 
     @property
     def num_tokens(self) -> int:
@@ -101,6 +102,11 @@ SPECS: dict[str, WorkloadSpec] = {
     "qwen3_30b_a3b_fp8": WorkloadSpec(
         "qwen3_30b_a3b_fp8", 2, 8, 1024, 2048, 128, 8, 768, "bf16", "fp8", 1.2, False,
         RoutingMode("softmax", True, "output"),
+    ),
+    # and with the experts' inputs quantised as well: both products on the fp8 matrix pipe
+    "qwen3_30b_a3b_w8a8": WorkloadSpec(
+        "qwen3_30b_a3b_w8a8", 2, 8, 1024, 2048, 128, 8, 768, "bf16", "fp8", 1.2, False,
+        RoutingMode("softmax", True, "output"), "mxfp8",
     ),
     "qwen3_decode_fp8": WorkloadSpec(
         "qwen3_decode_fp8", 4, 64, 1, 2048, 128, 8, 768, "bf16", "fp8", 1.2, False,
@@ -241,11 +247,12 @@ def small_spec(
     zipf_s: float | None = None,
     shared: bool = False,
     mode: RoutingMode = _REFERENCE_MODE,
+    act_quant: str | None = None,
 ) -> WorkloadSpec:
     """A free-form spec for tests at sizes the CPU evaluates in milliseconds."""
     return WorkloadSpec(
         "custom", seed, 1, tokens, model_dim, num_experts, top_k, inner_dim, dtype,
-        weight_dtype or dtype, zipf_s, shared, mode,
+        weight_dtype or dtype, zipf_s, shared, mode, act_quant,
     )
 
 
@@ -276,7 +283,7 @@ def build_module(wl: Workload, device, tile_m: int = 16):
             s.model_dim, s.inner_dim, s.shared, s.num_experts, 1.0, s.top_k,
             inner_dim_scale=1.0, auto_scale=False,
             score_fn=s.mode.score_fn, renormalize=s.mode.renormalize, scale_on=s.mode.scale_on,
-            router_bias=wl.router_bias is not None, tile_m=tile_m,
+            router_bias=wl.router_bias is not None, tile_m=tile_m, act_quant=s.act_quant,
         )
     finally:
         torch.set_default_dtype(prev)
