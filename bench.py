@@ -415,7 +415,10 @@ def main() -> int:
         work["experts"]["bytes"] / (HBM_PEAK_GBS * 1e9)
         > work["experts"]["flops"] / (MFMA_PEAK_TFLOPS[spec.dtype] * 1e12)
     )
-    peak_tf = MFMA_PEAK_TFLOPS[spec.dtype]
+    w8a8 = spec.act_quant == "mxfp8" and module.experts.runs_w8a8(dt, spec.num_tokens * spec.top_k)
+    # the matrix pipe the expert products run on: fp8 only when both operands are e4m3 (W8A8);
+    # e4m3 weights alone are turned into bf16 on the way to LDS
+    peak_tf = MFMA_PEAK_TFLOPS["fp8" if w8a8 else spec.dtype]
     fused_gather = bool(stage_ms.pop("fused_gather", False))
     t, d, k, b = spec.num_tokens, spec.model_dim, spec.top_k, elem_bytes(spec.dtype)
     work["dispatch_with_gather"] = dict(work["dispatch"])
@@ -429,14 +432,18 @@ def main() -> int:
         w = work[name]
         if name == "shared" or (name == "experts" and not experts_hbm_bound):
             tf = w["flops"] / (ms * 1e-3) / 1e12
-            ent.update(bound="mfma", achieved_tflops=round(tf, 2), frac=round(tf / peak_tf, 4))
+            pk = MFMA_PEAK_TFLOPS[spec.dtype] if name == "shared" else peak_tf
+            ent.update(bound="mfma", achieved_tflops=round(tf, 2), frac=round(tf / pk, 4))
         else:
             gbs = w["bytes"] / (ms * 1e-3) / 1e9
             ent.update(bound="hbm", achieved_gbs=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 4))
         stages[name] = ent
 
     exp_ms = stage_ms["experts"]
-    if spec.weight_dtype == "fp8" and experts_hbm_bound:
+    if w8a8:
+        kernel = ("glu_gemm_mx_kernel<gate,up> + <down> (fs2moe_grouped_swiglu_w8a8; the launch time "
+                  "includes mx_quantize_kernel over the token rows)")
+    elif spec.weight_dtype == "fp8" and experts_hbm_bound:
         kernel = "glu_gemm_fp8w_kernel<gate,up> + <down> (fs2moe_grouped_swiglu)"
     elif spec.weight_dtype == "fp8":
         # e4m3 weights turned into bf16 on the way to LDS: the matrix pipe runs in bf16
@@ -479,7 +486,8 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": spec.dtype if spec.weight_dtype != "fp8" else "bf16 activations, fp8 (e4m3) weights",
+        "dtype": ("fp8 (e4m3) expert products: block-scaled activations, per-channel-scaled weights; bf16 elsewhere"
+                  if w8a8 else spec.dtype if spec.weight_dtype != "fp8" else "bf16 activations, fp8 (e4m3) weights"),
         "data": "synthetic",
         "config": {
             "workload": spec.name,
