@@ -20,7 +20,7 @@ ABI_VERSION = 13
 F32, BF16, FP8_E4M3 = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
 W_IN_OUT, W_OUT_IN = 0, 1
-MAX_EXPERTS, MAX_TOP_K = 256, 16
+MAX_EXPERTS, MAX_TOP_K = 512, 32
 
 # name -> (restype, argtypes); mirrors include/fs2moe.h one to one
 _PROTOTYPES = {

@@ -155,6 +155,7 @@ static int launch_combine(const void* ye, const int32_t* inv_perm, const int32_t
   FS2_COMBINE_CASE(4)
   FS2_COMBINE_CASE(8)
   FS2_COMBINE_CASE(16)
+  FS2_COMBINE_CASE(32)
 #undef FS2_COMBINE_CASE
   set_error("combine: K=%d exceeds %d", K, FS2MOE_MAX_TOP_K);
   return FS2MOE_ERR_UNSUPPORTED;

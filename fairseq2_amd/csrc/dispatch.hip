@@ -14,20 +14,22 @@ namespace fs2moe {
 // The experts of token t, -1 where there is none (t past T, k past K, an index outside [0, E)).
 // Every load is issued, from an address inside the array, before any result is looked at: a load
 // behind a condition is waited for on the spot, one round trip per k.
+// KCAP: a compile-time bound on K (16 covers every published layer; 32 is the library's limit).
+template <int KCAP>
 __device__ __forceinline__ void load_token_experts(const int32_t* __restrict__ topk_idx, int t,
-                                                   int T, int K, int E,
-                                                   int (&ek)[FS2MOE_MAX_TOP_K]) {
+                                                   int T, int K, int E, int (&ek)[KCAP]) {
   const bool has_token = t < T;
   const int32_t* mine = topk_idx + (has_token ? (size_t)t * K : 0);
 #pragma unroll
-  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) ek[k] = mine[k < K ? k : 0];
+  for (int k = 0; k < KCAP; ++k) ek[k] = mine[k < K ? k : 0];
 #pragma unroll
-  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) {
+  for (int k = 0; k < KCAP; ++k) {
     const int e = ek[k];
     ek[k] = (has_token && k < K && e >= 0 && e < E) ? e : -1;
   }
 }
 
+template <int KCAP>
 __global__ __launch_bounds__(kDispTok) void dispatch_count_kernel(
     const int32_t* __restrict__ topk_idx, int T, int K, int E, int32_t* __restrict__ block_counts,
     int32_t* __restrict__ rank) {
@@ -41,10 +43,10 @@ __global__ __launch_bounds__(kDispTok) void dispatch_count_kernel(
   const int word = tid >> 5;
   const uint32_t bit = 1u << (tid & 31);
   // the token's experts stay in registers between the two passes
-  int ek[FS2MOE_MAX_TOP_K];
-  load_token_experts(topk_idx, t, T, K, E, ek);
+  int ek[KCAP];
+  load_token_experts<KCAP>(topk_idx, t, T, K, E, ek);
 #pragma unroll
-  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k)
+  for (int k = 0; k < KCAP; ++k)
     if (ek[k] >= 0) atomicOr(&s_bits[ek[k] * kDispWords + word], bit);
   __syncthreads();
   for (int i = tid; i < E * kDispWords; i += kDispTok) {
@@ -55,7 +57,7 @@ __global__ __launch_bounds__(kDispTok) void dispatch_count_kernel(
   }
   __syncthreads();
 #pragma unroll
-  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) {
+  for (int k = 0; k < KCAP; ++k) {
     if (k < K && t < T) {
       int r = 0;
       if (ek[k] >= 0) {
@@ -71,44 +73,50 @@ __global__ __launch_bounds__(kDispTok) void dispatch_count_kernel(
   }
 }
 
-// One block of 256 threads (E <= 256).  Turns per-block counts into per-block exclusive prefixes (in
-// place), and writes counts and the tile-padded offsets (a block-wide exclusive scan).
+// One block of 256 threads, the experts 256 at a time (one per thread, the rows of the rounds before
+// carried along).  Turns per-block counts into per-block exclusive prefixes (in place), and writes
+// counts and the tile-padded offsets (a block-wide exclusive scan).
 __global__ __launch_bounds__(256) void dispatch_scan_kernel(int32_t* __restrict__ block_counts,
                                                             int num_blocks, int E, int tile_m,
                                                             int32_t* __restrict__ counts,
                                                             int32_t* __restrict__ offsets) {
-  __shared__ int32_t s_wave_tot[4];
+  __shared__ int32_t s_wave_tot[2][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  int padded = 0;
-  if (tid < E) {
-    // chunks of 8 blocks: the loads of a chunk are independent of its stores and go out together
-    int run = 0;
-    for (int b0 = 0; b0 < num_blocks; b0 += 8) {
-      int c[8];
+  int carried = 0;
+  for (int e0 = 0; e0 < E; e0 += 256) {
+    const int ex = e0 + tid, par = (e0 >> 8) & 1;
+    int padded = 0;
+    if (ex < E) {
+      // chunks of 8 blocks: the loads of a chunk are independent of its stores and go out together
+      int run = 0;
+      for (int b0 = 0; b0 < num_blocks; b0 += 8) {
+        int c[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        c[i] = b0 + i < num_blocks ? block_counts[(size_t)(b0 + i) * E + tid] : 0;
+        for (int i = 0; i < 8; ++i)
+          c[i] = b0 + i < num_blocks ? block_counts[(size_t)(b0 + i) * E + ex] : 0;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if (b0 + i < num_blocks) block_counts[(size_t)(b0 + i) * E + tid] = run;
-        run += c[i];
+        for (int i = 0; i < 8; ++i) {
+          if (b0 + i < num_blocks) block_counts[(size_t)(b0 + i) * E + ex] = run;
+          run += c[i];
+        }
       }
+      counts[ex] = run;
+      padded = (run + tile_m - 1) / tile_m * tile_m;
     }
-    counts[tid] = run;
-    padded = (run + tile_m - 1) / tile_m * tile_m;
-  }
-  int incl = padded;
+    int incl = padded;
 #pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    int v = __shfl_up(incl, off, kWave);
-    if (lane >= off) incl += v;
+    for (int off = 1; off < 64; off <<= 1) {
+      int v = __shfl_up(incl, off, kWave);
+      if (lane >= off) incl += v;
+    }
+    if (lane == 63) s_wave_tot[par][wave] = incl;
+    __syncthreads();
+    int base = carried;
+    for (int w = 0; w < wave; ++w) base += s_wave_tot[par][w];
+    if (ex < E) offsets[ex] = base + incl - padded;
+    if (ex == E - 1) offsets[E] = base + incl;
+    for (int w = 0; w < 4; ++w) carried += s_wave_tot[par][w];
   }
-  if (lane == 63) s_wave_tot[wave] = incl;
-  __syncthreads();
-  int base = 0;
-  for (int w = 0; w < wave; ++w) base += s_wave_tot[w];
-  if (tid < E) offsets[tid] = base + incl - padded;
-  if (tid == E - 1) offsets[E] = base + incl;
 }
 
 template <typename TA>
@@ -222,13 +230,14 @@ __global__ __launch_bounds__(256) void dispatch_index_kernel(
 // All of dispatch for at most 256 tokens when no rows are copied (xe == NULL): count, scan and
 // index in one block.  A decode step spends more on starting three kernels than on their work.
 // Same arithmetic as the three kernels above, so the results are identical.
+template <int KCAP>
 __global__ __launch_bounds__(kDispTok) void dispatch_small_kernel(
     const int32_t* __restrict__ topk_idx, int T, int K, int E, int tile_m, int64_t max_rows,
     int32_t* __restrict__ counts, int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
     int32_t* __restrict__ inv_perm) {
   extern __shared__ uint32_t s_mem[];
   __shared__ int32_t s_wave_tot[4];
-  dispatch_small_block(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm, s_mem,
+  dispatch_small_block<KCAP>(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm, s_mem,
                        s_wave_tot, threadIdx.x, kDispTok);
 }
 
@@ -237,7 +246,7 @@ __global__ __launch_bounds__(kDispTok) void dispatch_small_kernel(
 // starting three kernels), block 0 writes it to memory, and then the blocks do what
 // dispatch_permute_kernel's do: blocks [0, pair_blocks) copy (and scale) a pair's row per wave,
 // block pair_blocks + e zero-fills the padding rows of expert e.  Same arithmetic, same results.
-template <typename TA>
+template <typename TA, int KCAP>
 __global__ __launch_bounds__(kDispTok) void dispatch_small_copy_kernel(
     const int32_t* __restrict__ topk_idx, const float* __restrict__ topk_w,
     const TA* __restrict__ x, int T, int K, int E, int D, int tile_m, int scale_input,
@@ -246,8 +255,8 @@ __global__ __launch_bounds__(kDispTok) void dispatch_small_copy_kernel(
     TA* __restrict__ xe) {
   extern __shared__ uint32_t s_mem[];
   __shared__ int32_t s_wave_tot[4];
-  dispatch_small_block(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm, s_mem,
-                       s_wave_tot, threadIdx.x, kDispTok, blockIdx.x == 0);
+  dispatch_small_block<KCAP>(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm,
+                             s_mem, s_wave_tot, threadIdx.x, kDispTok, blockIdx.x == 0);
   const uint32_t* s_bits = s_mem;
   const uint32_t* s_pref = s_mem + E * kDispWords;
   const int32_t* s_off = reinterpret_cast<const int32_t*>(s_pref + E * kDispWords);
@@ -326,31 +335,45 @@ extern "C" int fs2moe_dispatch(const int32_t* topk_idx, const float* topk_w, con
   int32_t* block_counts = static_cast<int32_t*>(workspace);
   int32_t* rank = block_counts + (size_t)nb * E;
 
-  if (nb == 1 && xe == nullptr) {
-    hipLaunchKernelGGL(dispatch_small_kernel, dim3(1), dim3(kDispTok),
-                       dispatch_small_lds_words(E) * sizeof(uint32_t), s, topk_idx, T, K, E,
-                       tile_m, max_rows, counts, offsets, perm, inv_perm);
+  // (the one-block forms scan the experts with a thread each: up to 256 of them)
+  const bool small = nb == 1 && E <= kDispTok;
+  if (small && xe == nullptr) {
+    const size_t lds = dispatch_small_lds_words(E) * sizeof(uint32_t);
+    if (K <= 16)
+      hipLaunchKernelGGL(dispatch_small_kernel<16>, dim3(1), dim3(kDispTok), lds, s, topk_idx, T, K,
+                         E, tile_m, max_rows, counts, offsets, perm, inv_perm);
+    else
+      hipLaunchKernelGGL(dispatch_small_kernel<FS2MOE_MAX_TOP_K>, dim3(1), dim3(kDispTok), lds, s,
+                         topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm);
     return check_launch("dispatch_small");
   }
-  if (nb == 1) {
+  if (small) {
     // (xe is given: the copying form of the same)
     const unsigned pair_blocks = (unsigned)(((int64_t)T * K + 3) / 4);
     const dim3 grid(pair_blocks + (unsigned)E), block(kDispTok);
     const size_t lds = dispatch_small_lds_words(E) * sizeof(uint32_t);
-    if (act_dtype == FS2MOE_F32)
-      hipLaunchKernelGGL(dispatch_small_copy_kernel<float>, grid, block, lds, s, topk_idx, topk_w,
-                         static_cast<const float*>(x), T, K, E, D, tile_m, scale_input, max_rows,
-                         pair_blocks, counts, offsets, perm, inv_perm, static_cast<float*>(xe));
-    else
-      hipLaunchKernelGGL(dispatch_small_copy_kernel<uint16_t>, grid, block, lds, s, topk_idx, topk_w,
-                         static_cast<const uint16_t*>(x), T, K, E, D, tile_m, scale_input, max_rows,
-                         pair_blocks, counts, offsets, perm, inv_perm, static_cast<uint16_t*>(xe));
+#define FS2_SMALL_COPY(TA, KC)                                                                       \
+  hipLaunchKernelGGL((dispatch_small_copy_kernel<TA, KC>), grid, block, lds, s, topk_idx, topk_w,    \
+                     static_cast<const TA*>(x), T, K, E, D, tile_m, scale_input, max_rows,           \
+                     pair_blocks, counts, offsets, perm, inv_perm, static_cast<TA*>(xe))
+    if (act_dtype == FS2MOE_F32) {
+      if (K <= 16) FS2_SMALL_COPY(float, 16);
+      else FS2_SMALL_COPY(float, FS2MOE_MAX_TOP_K);
+    } else {
+      if (K <= 16) FS2_SMALL_COPY(uint16_t, 16);
+      else FS2_SMALL_COPY(uint16_t, FS2MOE_MAX_TOP_K);
+    }
+#undef FS2_SMALL_COPY
     return check_launch("dispatch_small_copy");
   }
   if (nb > 0) {
-    hipLaunchKernelGGL(dispatch_count_kernel, dim3(nb), dim3(kDispTok),
-                       (size_t)E * kDispWords * 2 * sizeof(uint32_t), s, topk_idx, T, K, E,
-                       block_counts, rank);
+    const size_t lds = (size_t)E * kDispWords * 2 * sizeof(uint32_t);
+    if (K <= 16)
+      hipLaunchKernelGGL(dispatch_count_kernel<16>, dim3(nb), dim3(kDispTok), lds, s, topk_idx, T, K,
+                         E, block_counts, rank);
+    else
+      hipLaunchKernelGGL(dispatch_count_kernel<FS2MOE_MAX_TOP_K>, dim3(nb), dim3(kDispTok), lds, s,
+                         topk_idx, T, K, E, block_counts, rank);
     if (int rc = check_launch("dispatch_count")) return rc;
   }
   hipLaunchKernelGGL(dispatch_scan_kernel, dim3(1), dim3(256), 0, s, block_counts, nb, E, tile_m,

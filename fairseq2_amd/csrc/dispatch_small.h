@@ -17,9 +17,11 @@ __host__ __device__ inline size_t dispatch_small_lds_words(int E) {
 }
 
 // write: the results go to memory (else they are only left in LDS: s_bits, s_pref, s_off at s_mem).
+// KCAP: a compile-time bound on K.  E <= 256 (a thread per expert in the scan).
 // Called by every thread of a block of `nthreads` >= 256 threads (a multiple of 64); threads 0..255
 // are the tokens' threads, the others only help with the loops over LDS and pass the barriers.
 // topk_idx may have been written by this block before a barrier.
+template <int KCAP>
 __device__ __forceinline__ void dispatch_small_block(
     const int32_t* topk_idx, int T, int K, int E, int tile_m, int64_t max_rows, int32_t* counts,
     int32_t* offsets, int32_t* perm, int32_t* inv_perm, uint32_t* s_mem, int32_t* s_wave_tot,
@@ -33,11 +35,11 @@ __device__ __forceinline__ void dispatch_small_block(
   // The token's experts, loaded first and unconditionally (from the first token's where this thread
   // has no token or k is past K), so that all the loads are in flight together behind the clearing
   // of the bitmaps; what does not count is set to -1 afterwards.
-  int ek[FS2MOE_MAX_TOP_K];
+  int ek[KCAP];
   {
     const int32_t* mine = topk_idx + (has_token ? (size_t)t * K : 0);
 #pragma unroll
-    for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k)
+    for (int k = 0; k < KCAP; ++k)
       ek[k] = mine[k < K ? k : 0];
   }
   for (int i = tid; i < E * kDispWords; i += nthreads) s_bits[i] = 0u;
@@ -45,7 +47,7 @@ __device__ __forceinline__ void dispatch_small_block(
   const int word = tid >> 5;
   const uint32_t bit = 1u << (tid & 31);
 #pragma unroll
-  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) {
+  for (int k = 0; k < KCAP; ++k) {
     const int e = ek[k];
     ek[k] = (has_token && k < K && e >= 0 && e < E) ? e : -1;
     if (ek[k] >= 0) atomicOr(&s_bits[ek[k] * kDispWords + word], bit);
@@ -89,7 +91,7 @@ __device__ __forceinline__ void dispatch_small_block(
   if (!write) return;
   // pairs
 #pragma unroll
-  for (int k = 0; k < FS2MOE_MAX_TOP_K; ++k) {
+  for (int k = 0; k < KCAP; ++k) {
     if (k < K && t < T && tid < kDispTok) {
       const size_t p = (size_t)t * K + k;
       if (ek[k] < 0) {

@@ -406,7 +406,8 @@ static bool dma_offsets_fit(int64_t rows_bound, int D, int F) {
 #define FS2MOE_GEMV_MAX_ROWS 4
 #endif
 static bool gemv_applies(int act_dtype, int D, int F, const Groups& g, int rows_hint) {
-  if (act_dtype != FS2MOE_BF16 || g.counts == nullptr || rows_hint < 1 ||
+  // (the stream kernels find their expert with four ballots over the counts: up to 256 experts)
+  if (act_dtype != FS2MOE_BF16 || g.counts == nullptr || g.E > 256 || rows_hint < 1 ||
       rows_hint > FS2MOE_GEMV_MAX_ROWS)
     return false;
   const int r = rows_hint <= 1 ? 1 : rows_hint <= 2 ? 2 : 4;
@@ -454,8 +455,8 @@ static int launch_gemv_pair_r(const void* x, const int32_t* row_map, const Group
 #define FS2MOE_GEMV16_MAX_ROWS 16
 #endif
 static bool gemv16_applies(int act_dtype, int D, int F, const Groups& g, int rows_hint) {
-  if (act_dtype != FS2MOE_BF16 || g.counts == nullptr || rows_hint <= FS2MOE_GEMV_MAX_ROWS ||
-      rows_hint > FS2MOE_GEMV16_MAX_ROWS)
+  if (act_dtype != FS2MOE_BF16 || g.counts == nullptr || g.E > 256 ||
+      rows_hint <= FS2MOE_GEMV_MAX_ROWS || rows_hint > FS2MOE_GEMV16_MAX_ROWS)
     return false;
   return gemv16::offsets_fit(D, F) && gemv16::fits(D > F ? D : F, 8);
 }
@@ -663,11 +664,13 @@ static int grouped_swiglu_impl(const void* xe, const int32_t* row_map, const int
     // same matrix rate).  With few (decode) it is a stream over the weights: the kernels below.  The
     // row counts live on the device, so the choice goes by the mean number of rows per expert the
     // buffers are sized for.
-    if (max_rows / E >= kFp8GemmMinRowsPerExpert && dma_offsets_fit(max_rows, D, F)) {
+    // (the streaming kernels build their item table with a thread per expert: up to 256 experts)
+    if ((max_rows / E >= kFp8GemmMinRowsPerExpert || E > 256) && dma_offsets_fit(max_rows, D, F)) {
       Groups g{counts, offsets, E, 0};
       return launch_dma_pair<dma::W_FP8_TILED>(xe, row_map, g, max_rows, w_gate, w_up, w_down, s_gate,
                                                s_up, s_down, D, F, h, ye, st);
     }
+    FS2_REQUIRE(E <= 256, "grouped_swiglu: the e4m3 streaming kernels take up to 256 experts (E=%d)", E);
     // Persistent blocks, three or four per CU (what the kernels' registers allow), walking work
     // items.
     // A long K is split over the 4 waves of a block (the chain of dependent loads per wave sets the

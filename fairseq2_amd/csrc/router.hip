@@ -266,7 +266,10 @@ __global__ __launch_bounds__(kNormRows* kWave) void rms_norm_kernel(const TA* x,
 
 constexpr int kRouterTok = 8;     // tokens per wave
 constexpr int kRouterWaves = 4;   // waves per block
-constexpr int kRouterChunk = 64;  // rows of the router matrix staged at a time
+// rows of the router matrix staged at a time: 64 (one per lane of the token rows' loads) while the
+// f32 stage fits the 64 KB of static LDS, i.e. up to 256 experts, else 32
+template <int J>
+constexpr int router_chunk() { return J <= 4 ? 64 : 32; }
 
 template <typename TA, int J>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_fma_kernel(
@@ -274,6 +277,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_fma_kernel(
     const float* __restrict__ bias, int T, int D, int E, int K, int score_fn, int renorm,
     int32_t* __restrict__ topk_idx, float* __restrict__ topk_w, float* __restrict__ logits) {
   constexpr int EP = 64 * J;
+  constexpr int kRouterChunk = router_chunk<J>();
   __shared__ float s_r[kRouterChunk * EP];
 
   const int lane = lane_id();
@@ -307,7 +311,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_fma_kernel(
 #pragma unroll
     for (int i = 0; i < kRouterTok; ++i) {
       int t = t0 + i, d = d0 + lane;
-      xv[i] = (t < T && d < D) ? Elem<TA>::load(x + (size_t)t * D + d) : 0.f;
+      xv[i] = (t < T && d < D && lane < kRouterChunk) ? Elem<TA>::load(x + (size_t)t * D + d) : 0.f;
     }
 #pragma unroll
     for (int dd = 0; dd < kRouterChunk; ++dd) {
@@ -636,8 +640,9 @@ __global__ __launch_bounds__(kFinishDispatchThreads) void router_finish_dispatch
     select_topk<J>(v, lane, t, E, K, score_fn, renorm, topk_idx, topk_w);
   }
   __syncthreads();  // the tokens' experts are written and visible to the block
-  dispatch_small_block(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm, s_mem,
-                       s_wave_tot, threadIdx.x, kFinishDispatchThreads);
+  // (the host sends K > 16 through router_finish_kernel and the dispatch kernels instead)
+  dispatch_small_block<16>(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm,
+                           s_mem, s_wave_tot, threadIdx.x, kFinishDispatchThreads);
 }
 
 // ------------------------------------------------------------------------------------ f32 / MFMA
@@ -845,6 +850,10 @@ static int launch_router_fma(const void* x, const void* norm_w, float norm_eps, 
     FS2_ROUTER_CASE(2)
     FS2_ROUTER_CASE(3)
     FS2_ROUTER_CASE(4)
+    FS2_ROUTER_CASE(5)
+    FS2_ROUTER_CASE(6)
+    FS2_ROUTER_CASE(7)
+    FS2_ROUTER_CASE(8)
     default:
       set_error("router: E=%d exceeds %d", E, FS2MOE_MAX_EXPERTS);
       return FS2MOE_ERR_UNSUPPORTED;
@@ -864,7 +873,7 @@ constexpr int kNormAloneMaxTokens = 4096;
 // How many blocks share a 32-token tile of the bf16 MFMA router: enough to put about 256 blocks on
 // the chip, each with at least one step of its k-groups, at most 8.  1 = no split.
 static int router_slices(int T, int D, int E, int act_dtype) {
-  if (act_dtype != FS2MOE_BF16 || D % 8 != 0 || E % 8 != 0 || T < 1) return 1;
+  if (act_dtype != FS2MOE_BF16 || D % 8 != 0 || E % 8 != 0 || E > 256 || T < 1) return 1;
   const int tiles = (T + rmfma::BT - 1) / rmfma::BT;
   const int groups = E <= 128 ? rmfma::Shape<1>::GROUPS : rmfma::Shape<2>::GROUPS;
   const int nk = (D + 63) / 64;
@@ -903,7 +912,7 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
   hipStream_t s = static_cast<hipStream_t>(stream);
   // (a single token tile of the bf16 MFMA router normalises in its own blocks, also when several
   // blocks share the tile: one launch fewer for a decode step)
-  const bool one_tile = act_dtype == FS2MOE_BF16 && T <= rmfma::BT && D % 8 == 0 && E % 8 == 0 &&
+  const bool one_tile = act_dtype == FS2MOE_BF16 && T <= rmfma::BT && D % 8 == 0 && E % 8 == 0 && E <= 256 &&
                         aligned16(x) && aligned16(router) && aligned16(xn);
   if (xn != nullptr && T <= kNormAloneMaxTokens && !one_tile) {
     // few token blocks: normalise with the whole chip first, then route xn as it is
@@ -940,8 +949,9 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
     return launch_router_fma<float>(x, norm_w, norm_eps, xn, router, bias, T, D, E, K, score_fn, renormalize, topk_idx,
                                     topk_w, logits, s);
   }
-  // The MFMA path moves 16-byte chunks: D and E multiples of 8 and aligned bases.
-  if (D % 8 == 0 && E % 8 == 0 && aligned16(x) && aligned16(router)) {
+  // The MFMA path moves 16-byte chunks (D and E multiples of 8, aligned bases) and holds up to 256
+  // experts; anything else takes the FMA kernel.
+  if (D % 8 == 0 && E % 8 == 0 && E <= 256 && aligned16(x) && aligned16(router)) {
     dim3 grid((T + rmfma::BT - 1) / rmfma::BT);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const uint16_t* rp = static_cast<const uint16_t*>(router);
@@ -980,7 +990,7 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
       if (int rc = check_launch("router_mfma (split)")) return rc;
       const dim3 fgrid((T + 3) / 4), fblock(4 * kWave);
       const int j = (E + 63) / 64;
-      if (disp != nullptr && logits == nullptr && T <= kFinishDispatchTokens) {
+      if (disp != nullptr && logits == nullptr && T <= kFinishDispatchTokens && K <= 16) {
         const size_t dlds = dispatch_small_lds_words(E) * sizeof(uint32_t);
 #define FS2_FINISH_CASE(JJ)                                                                       \
   case JJ:                                                                                        \

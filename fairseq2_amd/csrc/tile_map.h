@@ -22,78 +22,34 @@ __device__ __forceinline__ bool locate_tile(const Groups& g, int mt, int& e, int
     row_end = g.dense_rows;
     return row0 < row_end;
   }
-  __shared__ int s_wave_tot[4];
+  __shared__ int s_wave_tot[2][4];
   __shared__ int s_tile[3];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int cnt = tid < g.E ? g.counts[tid] : 0;
-  const int tiles = (cnt + BM - 1) / BM;
-  int incl = tiles;
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    int v = __shfl_up(incl, off, kWave);
-    if (lane >= off) incl += v;
-  }
-  if (lane == 63) s_wave_tot[wave] = incl;
   if (tid == 0) s_tile[0] = -1;
-  __syncthreads();
-  int base = 0;
-  for (int w = 0; w < wave; ++w) base += s_wave_tot[w];
-  const int excl = base + incl - tiles;
-  if (tiles > 0 && mt >= excl && mt < excl + tiles) {
-    const int off = g.offsets[tid];
-    s_tile[0] = tid;
-    s_tile[1] = off + (mt - excl) * BM;
-    s_tile[2] = off + cnt;
-  }
-  __syncthreads();
-  e = s_tile[0];
-  row0 = s_tile[1];
-  row_end = s_tile[2];
-  return e >= 0;
-}
-
-// Maps a block to an output tile with an XCD-aware order.  Workgroups are dealt round-robin to the
-// eight XCDs (block b runs on XCD b % 8), each with its own L2.  Tiles are numbered m-tile major,
-// n-tile minor, and XCD c takes the contiguous range [c * per, (c + 1) * per) of them, so the
-// blocks resident on one XCD work on neighbouring tiles and share activation slabs (same m-tile)
-// and weight slabs (same expert and n-tile) through that XCD's L2.  The number of real tiles is
-// data dependent and computed here from counts; surplus blocks return false.
-template <int BM, int NWAVES>
-__device__ __forceinline__ bool map_block(const Groups& g, int n_tiles, int& e, int& row0,
-                                          int& row_end, int& nt) {
-  __shared__ int s_wave_tot[NWAVES];
-  __shared__ int s_tile[3];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const bool dense = g.counts == nullptr;
-  const int cnt = dense ? (tid == 0 ? g.dense_rows : 0) : (tid < g.E ? g.counts[tid] : 0);
-  const int tiles = (cnt + BM - 1) / BM;
-  int incl = tiles;
+  // the experts 256 at a time (one per thread), carrying the tiles of the rounds before
+  int carried = 0;
+  for (int e0 = 0; e0 < g.E; e0 += 256) {
+    const int ex = e0 + tid, par = (e0 >> 8) & 1;
+    const int cnt = ex < g.E ? g.counts[ex] : 0;
+    const int tiles = (cnt + BM - 1) / BM;
+    int incl = tiles;
 #pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    int v = __shfl_up(incl, off, kWave);
-    if (lane >= off) incl += v;
-  }
-  if (lane == 63) s_wave_tot[wave] = incl;
-  if (tid == 0) s_tile[0] = -1;
-  __syncthreads();
-  int base = 0;
-  for (int w = 0; w < wave; ++w) base += s_wave_tot[w];
-  int total = 0;
-#pragma unroll
-  for (int w = 0; w < NWAVES; ++w) total += s_wave_tot[w];
-  const long long real = (long long)total * n_tiles;
-  const long long per = (real + 7) / 8;
-  const long long idx = blockIdx.x >> 3;
-  const long long logical = (long long)(blockIdx.x & 7) * per + idx;
-  if (idx >= per || logical >= real) return false;  // block-uniform
-  const int mt = (int)(logical / n_tiles);
-  nt = (int)(logical - (long long)mt * n_tiles);
-  const int excl = base + incl - tiles;
-  if (tiles > 0 && mt >= excl && mt < excl + tiles) {
-    const int off = dense ? 0 : g.offsets[tid];
-    s_tile[0] = tid;
-    s_tile[1] = off + (mt - excl) * BM;
-    s_tile[2] = off + cnt;
+    for (int off = 1; off < 64; off <<= 1) {
+      int v = __shfl_up(incl, off, kWave);
+      if (lane >= off) incl += v;
+    }
+    if (lane == 63) s_wave_tot[par][wave] = incl;
+    __syncthreads();
+    int base = carried;
+    for (int w = 0; w < wave; ++w) base += s_wave_tot[par][w];
+    const int excl = base + incl - tiles;
+    if (tiles > 0 && mt >= excl && mt < excl + tiles) {
+      const int off = g.offsets[ex];
+      s_tile[0] = ex;
+      s_tile[1] = off + (mt - excl) * BM;
+      s_tile[2] = off + cnt;
+    }
+    for (int w = 0; w < 4; ++w) carried += s_wave_tot[par][w];
   }
   __syncthreads();
   e = s_tile[0];

@@ -42,8 +42,8 @@ extern "C" {
 #define FS2MOE_W_OUT_IN 1 /* (out, in), in contiguous: nn.Linear, the shared expert (ffn.py:302-347) */
 
 /* limits */
-#define FS2MOE_MAX_EXPERTS 256
-#define FS2MOE_MAX_TOP_K 16
+#define FS2MOE_MAX_EXPERTS 512
+#define FS2MOE_MAX_TOP_K 32
 
 /* bytes of the library's built-in scratch array (fs2moe_forward_static) */
 #define FS2MOE_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)

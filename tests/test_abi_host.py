@@ -177,8 +177,8 @@ def test_backward_entry_points_report_argument_errors_without_touching_the_gpu(l
     # element-wise and per-token steps
     rc = lib.fs2moe_swiglu_backward(fake, fake, fake, 10, 60, _abi.BF16, fake, fake, fake, None)
     assert rc == -1 and b"F=60" in err()
-    rc = lib.fs2moe_pair_dot(fake, None, fake, fake, 4, 17, 64, _abi.BF16, fake, None)
-    assert rc == -1 and b"K=17" in err()
+    rc = lib.fs2moe_pair_dot(fake, None, fake, fake, 4, 33, 64, _abi.BF16, fake, None)
+    assert rc == -1 and b"K=33" in err()
     rc = lib.fs2moe_router_backward(fake, fake, fake, fake, 4, 1000, 2, 0, 0, _abi.BF16, fake, None)
     assert rc == -1 and b"E=1000" in err()
     rc = lib.fs2moe_router_backward(fake, fake, fake, fake, 4, 8, 2, 5, 0, _abi.BF16, fake, None)

@@ -34,7 +34,9 @@ def _say(*a):
         (100, 512, 200, 16, "softmax_plain", 1.1),
         (64, 72, 5, 5, "sigmoid_renorm", None),  # K == E
         (31, 64, 1, 1, "reference", None),  # E == 1
-        (50, 128, 256, 16, "softmax_renorm", 1.0),  # the largest E and K the library takes
+        (50, 128, 256, 16, "softmax_renorm", 1.0),  # the largest E the matrix-pipe router takes
+        (70, 128, 512, 32, "softmax_renorm", 1.0),  # the largest E and K the library takes
+        (33, 200, 384, 24, "sigmoid_renorm", None),
         # bf16 with D >= 512 and few tokens: several blocks share a token tile
         (64, 2048, 128, 8, "softmax_renorm", 1.2),   # 8 blocks per tile
         (33, 1024, 256, 16, "softmax_plain", 1.0),   # two-fragment kernel, 8 blocks per tile

@@ -32,8 +32,8 @@ MODES = [
 def _draw(rng):
     dtype = rng.choice(["bf16", "bf16", "fp32"])
     wdt = "fp8" if (dtype == "bf16" and rng.random() < 0.3) else None
-    e = rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 24, 32, 40, 64, 72, 128, 136, 200, 256])
-    k = rng.randint(1, min(e, 16))
+    e = rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 24, 32, 40, 64, 72, 128, 136, 200, 256, 264, 384, 500, 512])
+    k = rng.randint(1, min(e, 32 if rng.random() < 0.25 else 16))
     t = rng.choice([1, 2, 7, 16, 17, 31, 32, 33, 64, 100, 255, 256, 257, 511, 600, 1100])
     aligned = wdt is not None or rng.random() < 0.7
     d = rng.choice([64, 128, 192, 256, 512]) if aligned else rng.choice([72, 136, 200])
@@ -54,6 +54,16 @@ FIXED = [
          tile_m=3, res=False),
     dict(dtype="bf16", wdt=None, e=200, k=11, t=600, d=192, f=64, mode=MODES[3], shared=True, zipf=1.0,
          tile_m=100, res=True),
+    # more experts and a larger top-k than any published layer (the reference takes any, moe.py:35-48):
+    # past 256 experts the router runs on the vector ALUs and the stream kernels stand aside
+    dict(dtype="bf16", wdt=None, e=384, k=24, t=600, d=256, f=128, mode=MODES[1], shared=False, zipf=1.0,
+         tile_m=16, res=False),
+    dict(dtype="bf16", wdt="fp8", e=512, k=32, t=257, d=128, f=192, mode=MODES[0], shared=True, zipf=None,
+         tile_m=3, res=True),
+    dict(dtype="fp32", wdt=None, e=300, k=17, t=7, d=72, f=40, mode=MODES[2], shared=False, zipf=1.5,
+         tile_m=1, res=False),
+    dict(dtype="bf16", wdt=None, e=500, k=20, t=9, d=256, f=128, mode=MODES[1], shared=False, zipf=None,
+         tile_m=16, res=False),
 ]
 
 
