@@ -136,7 +136,7 @@ _PROTOTYPES = {
     "fs2moe_mx_quantize": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p]),
     "fs2moe_grouped_swiglu_w8a8_supported": (c_int32, [c_int32, c_int32, c_int64]),
     "fs2moe_grouped_swiglu_w8a8": (
-        c_int32, [c_void_p] * 11 + [c_int32] * 3 + [c_int64] + [c_void_p] * 4,
+        c_int32, [c_void_p] * 11 + [c_int32] * 3 + [c_int64] * 2 + [c_void_p] * 4,
     ),
     "fs2moe_forward_norm": (
         c_int32,
@@ -467,16 +467,29 @@ def keeps_products(model_dim: int, inner_dim: int, rows: int, act_dtype: torch.d
 
 def mx_quantize(x: Tensor) -> tuple[Tensor, Tensor]:
     """bf16 rows ``(rows, D)`` -> e4m3 codes ``(rows, D)`` (as uint8) and one exponent byte per row
-    and 32 features ``(rows, D / 32)`` (``fs2moe_mx_quantize``)."""
+    and 32 features in the library's k-group-major layout ``(D / 128, rows, 4)``
+    (``fs2moe_mx_quantize``; :func:`mx_scales_row_major` gives ``(rows, D / 32)``)."""
     lib = load()
-    if x.dim() != 2 or x.dtype != torch.bfloat16 or x.shape[1] % 32:
-        raise ValueError("mx_quantize takes (rows, D) bf16 with D a multiple of 32")
+    if x.dim() != 2 or x.dtype != torch.bfloat16 or x.shape[1] % 128:
+        raise ValueError("mx_quantize takes (rows, D) bf16 with D a multiple of 128")
     rows, d = x.shape
     codes = torch.empty((rows, d), dtype=torch.uint8, device=x.device)
-    scales = torch.empty((rows, d // 32), dtype=torch.uint8, device=x.device)
+    scales = torch.empty((d // 128, rows, 4), dtype=torch.uint8, device=x.device)
     rc = lib.fs2moe_mx_quantize(_ptr(x), rows, d, _ptr(codes), _ptr(scales), _stream())
     _check(rc, "fs2moe_mx_quantize")
     return codes, scales
+
+
+def mx_scales_row_major(scales: Tensor) -> Tensor:
+    """Scale bytes ``(K / 128, rows, 4)`` as the library stores them -> ``(rows, K / 32)``."""
+    g, rows, four = scales.shape
+    return scales.permute(1, 0, 2).reshape(rows, g * four).contiguous()
+
+
+def mx_scales_k_major(scales: Tensor) -> Tensor:
+    """Scale bytes ``(rows, K / 32)`` -> the library's ``(K / 128, rows, 4)``."""
+    rows, nb = scales.shape
+    return scales.reshape(rows, nb // 4, 4).permute(1, 0, 2).contiguous()
 
 
 def w8a8_supported(model_dim: int, inner_dim: int, rows: int) -> bool:
@@ -497,12 +510,13 @@ def grouped_swiglu_w8a8(
 ) -> tuple[Tensor, Tensor, Tensor]:
     """The grouped SwiGLU network on the fp8 matrix pipe (``fs2moe_grouped_swiglu_w8a8``): block-scaled
     e4m3 rows (:func:`mx_quantize`) against tiled e4m3 weights with channel scales.  Returns
-    ``(ye, hq, hs)``: bf16 output rows and the quantised gated product."""
+    ``(ye, hq, hs)``: bf16 output rows and the quantised gated product (scales k-group major)."""
     lib = load()
     rows, d = xq.shape
+    x_rows = rows
     dev = xq.device
     _same("xq", xq, (rows, d), torch.uint8, dev)
-    _same("xs", xs, (rows, d // 32), torch.uint8, dev)
+    _same("xs", xs, (d // 128, rows, 4), torch.uint8, dev)
     if row_map is not None:
         if row_map.dtype != torch.int32 or row_map.dim() != 1:
             raise ValueError("row_map must be a 1-d int32 tensor")
@@ -517,12 +531,12 @@ def grouped_swiglu_w8a8(
     if [tuple(s.shape) for s in scales] != want or any(s.dtype != torch.float32 for s in scales):
         raise ValueError("fp8 scales must be f32 (E, F), (E, F), (E, D)")
     hq = torch.empty((rows, f), dtype=torch.uint8, device=dev)
-    hs = torch.empty((rows, f // 32), dtype=torch.uint8, device=dev)
+    hs = torch.empty((f // 128, rows, 4), dtype=torch.uint8, device=dev)
     ye = torch.empty((rows, d), dtype=torch.bfloat16, device=dev)
     rc = lib.fs2moe_grouped_swiglu_w8a8(
         _ptr(xq), _ptr(xs), _ptr(row_map), _ptr(counts), _ptr(offsets), _ptr(w_gate), _ptr(w_up),
-        _ptr(w_down), _ptr(scales[0]), _ptr(scales[1]), _ptr(scales[2]), num_experts, d, f, rows,
-        _ptr(hq), _ptr(hs), _ptr(ye), _stream(),
+        _ptr(w_down), _ptr(scales[0]), _ptr(scales[1]), _ptr(scales[2]), num_experts, d, f, x_rows,
+        rows, _ptr(hq), _ptr(hs), _ptr(ye), _stream(),
     )
     _check(rc, "fs2moe_grouped_swiglu_w8a8")
     return ye, hq, hs

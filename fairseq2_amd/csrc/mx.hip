@@ -21,7 +21,7 @@ static int mx_cu_count() {
 extern "C" int fs2moe_mx_quantize(const void* x, int64_t rows, int32_t D, void* codes, void* scales,
                                   void* stream) {
   FS2_REQUIRE(x && codes && scales, "mx_quantize: null pointer");
-  FS2_REQUIRE(rows >= 0 && D > 0 && D % 32 == 0, "mx_quantize: rows=%lld, D=%d (a multiple of 32)",
+  FS2_REQUIRE(rows >= 0 && D > 0 && D % 128 == 0, "mx_quantize: rows=%lld, D=%d (a multiple of 128)",
               (long long)rows, D);
   FS2_REQUIRE(aligned16(x) && aligned16(codes), "mx_quantize: buffers must be 16-byte aligned");
   if (rows == 0) return FS2MOE_OK;
@@ -47,8 +47,8 @@ extern "C" int fs2moe_grouped_swiglu_w8a8(const void* xq, const void* xs, const 
                                           const void* w_gate, const void* w_up, const void* w_down,
                                           const float* s_gate, const float* s_up,
                                           const float* s_down, int32_t E, int32_t D, int32_t F,
-                                          int64_t max_rows, void* hq, void* hs, void* ye,
-                                          void* stream) {
+                                          int64_t x_rows, int64_t max_rows, void* hq, void* hs,
+                                          void* ye, void* stream) {
   using namespace mx;
   FS2_REQUIRE(xq && xs && counts && offsets && w_gate && w_up && w_down && s_gate && s_up && s_down &&
                   hq && hs && ye,
@@ -57,6 +57,10 @@ extern "C" int fs2moe_grouped_swiglu_w8a8(const void* xq, const void* xs, const 
               FS2MOE_MAX_EXPERTS);
   FS2_REQUIRE(max_rows >= 0 && max_rows < (1ll << 31), "grouped_swiglu_w8a8: max_rows=%lld",
               (long long)max_rows);
+  // x_rows: the rows of xq / xs (their number places a k-group's scales): the token count with a
+  // row map, else max_rows
+  FS2_REQUIRE(x_rows >= 1 && x_rows < (1ll << 31) && (row_map != nullptr || x_rows == max_rows),
+              "grouped_swiglu_w8a8: x_rows=%lld", (long long)x_rows);
   FS2_REQUIRE(fs2moe_grouped_swiglu_w8a8_supported(D, F, max_rows),
               "grouped_swiglu_w8a8: D=%d and F=%d must be multiples of %d, and the operands "
               "addressable with 32-bit byte offsets",
@@ -67,6 +71,7 @@ extern "C" int fs2moe_grouped_swiglu_w8a8(const void* xq, const void* xs, const 
                   (reinterpret_cast<uintptr_t>(hs) & 3u) == 0,
               "grouped_swiglu_w8a8: buffers must be 16-byte aligned (scale bytes: 4)");
   if (max_rows == 0) return FS2MOE_OK;
+  FS2_REQUIRE(x_rows * (int64_t)D <= 0xffffffffll, "grouped_swiglu_w8a8: xq is addressed with 32-bit byte offsets");
   hipStream_t st = static_cast<hipStream_t>(stream);
   auto k1 = glu_gemm_mx_kernel<true>;
   auto k2 = glu_gemm_mx_kernel<false>;
@@ -100,12 +105,12 @@ extern "C" int fs2moe_grouped_swiglu_w8a8(const void* xq, const void* xs, const 
   hipLaunchKernelGGL(k1, dim3((unsigned)num_blocks), dim3(NWAVES * 64), SMEM_BYTES, st,
                      static_cast<const uint8_t*>(xq), static_cast<const uint8_t*>(xs), row_map,
                      static_cast<const uint8_t*>(w_gate), static_cast<const uint8_t*>(w_up), s_gate,
-                     s_up, hq, static_cast<uint8_t*>(hs), F, D, F, g, nt1);
+                     s_up, hq, static_cast<uint8_t*>(hs), F, D, F, g, nt1, (int)x_rows, (int)max_rows);
   if (int rc = check_launch("glu_gemm_mx<gate,up>")) return rc;
   hipLaunchKernelGGL(k2, dim3((unsigned)num_blocks), dim3(NWAVES * 64), SMEM_BYTES, st,
                      static_cast<const uint8_t*>(hq), static_cast<const uint8_t*>(hs),
                      static_cast<const int32_t*>(nullptr), static_cast<const uint8_t*>(w_down),
                      static_cast<const uint8_t*>(nullptr), s_down, static_cast<const float*>(nullptr),
-                     ye, static_cast<uint8_t*>(nullptr), D, F, D, g, nt2);
+                     ye, static_cast<uint8_t*>(nullptr), D, F, D, g, nt2, (int)max_rows, 0);
   return check_launch("glu_gemm_mx<down>");
 }

@@ -270,13 +270,18 @@ int fs2moe_forward_norm(const void* x, const void* norm_weight, float norm_eps,
  *     X = the smallest integer with max|block| / 2^X <= 448   (-127 for a zero block)
  *     code = e4m3(value / 2^X), round to nearest even         value ~ code * 2^X
  *
- * fs2moe_mx_quantize: x [rows, D] bf16 -> codes [rows, D] (1 byte each) and scales [rows, D / 32];
- *   D a multiple of 32.
+ * Scale bytes are stored k-group major, [features / 128][rows][4]: the four blocks of 128
+ * consecutive features of a row form one dword, and the dwords of consecutive rows are consecutive
+ * (what a kernel reads per step is exactly that dword of each of its rows).
+ *
+ * fs2moe_mx_quantize: x [rows, D] bf16 -> codes [rows, D] (1 byte each) and scales [D / 128][rows][4];
+ *   D a multiple of 128.
  * fs2moe_grouped_swiglu_w8a8: the grouped SwiGLU network of fs2moe_grouped_swiglu on such rows.
- *   xq [T or max_rows, D] codes, xs [.., D / 32] scales, both read through row_map [max_rows] when it
- *   is given (the gather of moe.py:131 fused into the first product), else expert-major;
- *   hq [max_rows, F] / hs [max_rows, F / 32]: the gated product, quantised the same way by the first
- *   kernel's epilogue (from its f32 values) and read by the second; ye [max_rows, D] bf16.
+ *   xq [x_rows, D] codes, xs [D / 128][x_rows][4] scales, both read through row_map [max_rows] when it
+ *   is given (the gather of moe.py:131 fused into the first product; x_rows = T), else expert-major
+ *   (x_rows = max_rows);
+ *   hq [max_rows, F] / hs [F / 128][max_rows][4]: the gated product, quantised the same way by the
+ *   first kernel's epilogue (from its f32 values) and read by the second; ye [max_rows, D] bf16.
  *   D and F multiples of 128 (fs2moe_grouped_swiglu_w8a8_supported says whether sizes qualify).
  */
 int fs2moe_mx_quantize(const void* x, int64_t rows, int32_t D, void* codes, void* scales,
@@ -286,8 +291,8 @@ int fs2moe_grouped_swiglu_w8a8(const void* xq, const void* xs, const int32_t* ro
                                const int32_t* counts, const int32_t* offsets, const void* w_gate,
                                const void* w_up, const void* w_down, const float* s_gate,
                                const float* s_up, const float* s_down, int32_t E, int32_t D,
-                               int32_t F, int64_t max_rows, void* hq, void* hs, void* ye,
-                               void* stream);
+                               int32_t F, int64_t x_rows, int64_t max_rows, void* hq, void* hs,
+                               void* ye, void* stream);
 
 /*
  * The whole layer without a workspace argument, for callers that cannot allocate device memory

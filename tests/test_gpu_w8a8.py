@@ -27,7 +27,7 @@ def _say(*a):
     print(*a, flush=True)
 
 
-@pytest.mark.parametrize("rows,d", [(1, 32), (7, 96), (300, 2048), (1025, 256)])
+@pytest.mark.parametrize("rows,d", [(1, 128), (7, 384), (300, 2048), (1025, 256)])
 def test_mx_quantize_matches_oracle_bit_for_bit(gpu_device, rows, d):
     _say("mx_quantize", rows, d)
     g = torch.Generator().manual_seed(rows + d)
@@ -39,7 +39,9 @@ def test_mx_quantize_matches_oracle_bit_for_bit(gpu_device, rows, d):
         x[2, 32:64] = 3.0e38  # the largest
     want_c, want_s = O.mx_quantize(x)
     got_c, got_s = _abi.mx_quantize(x.to(gpu_device))
-    assert torch.equal(got_s.cpu(), want_s)
+    assert got_s.shape == (d // 128, rows, 4)
+    assert torch.equal(_abi.mx_scales_row_major(got_s).cpu(), want_s)
+    assert torch.equal(_abi.mx_scales_k_major(want_s.to(gpu_device)), got_s)
     assert torch.equal(got_c.cpu(), want_c.view(torch.uint8))
 
 
@@ -89,11 +91,12 @@ def test_grouped_swiglu_w8a8_matches_oracle(gpu_device, rows, d, f, mapped):
     xq, xs = O.mx_quantize(src)
     pk = lambda name: _abi.pack_fp8_weights(wts[name][0].to(dev), e)  # noqa: E731
     ye, hq, hs = _abi.grouped_swiglu_w8a8(
-        xq.view(torch.uint8).to(dev), xs.to(dev), counts.to(dev), offsets.to(dev), pk("gate"), pk("up"), pk("down"),
+        xq.view(torch.uint8).to(dev), _abi.mx_scales_k_major(xs.to(dev)), counts.to(dev), offsets.to(dev), pk("gate"), pk("up"), pk("down"),
         tuple(wts[n][1].to(dev) for n in ("gate", "up", "down")), e,
         row_map=None if row_map is None else row_map.to(dev),
     )
     torch.cuda.synchronize()
+    hs_rows = _abi.mx_scales_row_major(hs).cpu()
     xr = O.mx_round(x_rows.double())
     for ex in range(e):
         lo, n = int(offsets[ex]), rows[ex]
@@ -102,7 +105,7 @@ def test_grouped_swiglu_w8a8_matches_oracle(gpu_device, rows, d, f, mapped):
         u = xr[lo : lo + n]
         wg, wu, wd = (wts[k][2].double().view(e, -1, wts[k][2].shape[1])[ex] for k in ("gate", "up", "down"))
         h_ref = torch.nn.functional.silu(u @ wg) * (u @ wu)
-        h_dev = O.mx_dequantize(hq[lo : lo + n].cpu().view(torch.float8_e4m3fn), hs[lo : lo + n].cpu()).double()
+        h_dev = O.mx_dequantize(hq[lo : lo + n].cpu().view(torch.float8_e4m3fn), hs_rows[lo : lo + n]).double()
         # the device's codes: the oracle's, or a neighbour where the f32 sum sat on a rounding boundary:
         # one e4m3 step, which is 2^-3 of the value at most in the normal range and 2^-9 of the block's
         # scale (at most 2^-16 of its largest element) below it; twice that if the block's largest
