@@ -30,16 +30,17 @@ MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3, "fp8": 5000.0}  # dense, publ
 # `--pmc WRITE_SIZE` runs of this script (see profiles/); None until measured for a workload.
 # The commit whose kernels the table below was measured on: a kernel change after it makes the
 # figures stale until the counter runs are repeated (the roofline object carries the stamp).
-MEASURED_TRAFFIC_AT = "6025f48"
+MEASURED_TRAFFIC_AT = "ffa7a90"
 MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
-    # profiles/bench_<workload>_all_kernels.md, the two launches of fs2moe_grouped_swiglu together
+    # profiles/bench_<workload>_all_kernels.md, the two launches of the grouped experts together
     # (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0 against a 256 MiB copy)
-    "qwen3_30b_a3b": 2.650e9,     # gate/up 1549 + 101 MB, down 729 + 270 MB
-    "mixtral_8x7b": 14.950e9,     # gate/up 10286 + 470 MB, down 4058 + 136 MB
-    "llama4_scout": 6.639e9,      # routed experts only: gate/up 4231 + 134 MB, down 2188 + 86 MB
-    "small_fp32": 0.862e9,        # gate/up 398 + 46 MB, down 401 + 17 MB
-    "qwen3_decode_fp8": 0.224e9,  # gate/up 142 + 1 MB, down 77 + 4 MB
-    "qwen3_30b_a3b_fp8": 1.895e9,  # gate/up 1035 + 101 MB, down 490 + 270 MB
+    "qwen3_30b_a3b": 2.626e9,     # gate/up 1538 + 101 MB, down 716 + 270 MB
+    "mixtral_8x7b": 14.773e9,     # gate/up 10123 + 470 MB, down 4045 + 136 MB
+    "llama4_scout": 6.624e9,      # routed experts only: gate/up 4244 + 134 MB, down 2161 + 86 MB
+    "small_fp32": 0.867e9,        # gate/up 404 + 46 MB, down 401 + 17 MB
+    "qwen3_decode_fp8": 0.220e9,  # gate/up 139 + 1 MB, down 75 + 5 MB
+    "qwen3_30b_a3b_fp8": 1.880e9,  # gate/up 1032 + 101 MB, down 478 + 270 MB
+    "qwen3_30b_a3b_w8a8": 1.465e9,  # gate/up 774 + 67 MB, down 355 + 269 MB
 }
 
 
