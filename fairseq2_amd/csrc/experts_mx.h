@@ -62,6 +62,15 @@ __device__ __forceinline__ uint32_t to_e4m3x4(float a, float b, float c, float d
 }
 }  // namespace mx
 
+// Which of a 1 KB weight tile's 16 channel rows lane l of a producer takes (with the 16 codes at
+// k 16 (l % 4) of it).  As fp8_tile_row in experts_dma.h, for this kernel's stores: a lane writes one
+// 16-byte chunk, four lanes the 64-byte half of a 128-byte LDS row, and the two rows served together
+// (eight lanes) must land in different halves: rows r and r + 8, whose swizzle keys differ by 4
+// (6.5 against 8.0 clocks per store instruction in the probe).
+__device__ __forceinline__ int mx_tile_row(int lane) {
+  return (((lane >> 2) & 1) << 3) | ((lane >> 3) & 7);
+}
+
 // A [a_rows, Kdim] e4m3 codes with scale bytes As, both read through row_map when it is given; B0 / B1
 // tiled e4m3 weights with channel scales S0 / S1 [E, N].
 // DUAL: C = e4m3 codes [c_rows, N] (ldc bytes per row) and their scale bytes Cs; else C = bf16.
@@ -243,7 +252,7 @@ __global__ __launch_bounds__(mx::NWAVES * 64) void glu_gemm_mx_kernel(
         const int gi = p >> 1, kb = p & 1;
         int group = t.n0 / 16 + (DUAL ? (gi & 7) : gi);
         group = group < N / 16 ? group : N / 16 - 1;  // clamped channels are never stored
-        pb[jj] = (uint32_t)(((size_t)group * nkb + kb) * 1024 + lane * 16);
+        pb[jj] = (uint32_t)(((size_t)group * nkb + kb) * 1024 + mx_tile_row(lane) * 64 + (lane & 3) * 16);
       }
     };
     u32x4 stage[16];
@@ -274,9 +283,9 @@ __global__ __launch_bounds__(mx::NWAVES * 64) void glu_gemm_mx_kernel(
       for (int jj = 0; jj < 8; ++jj)
         if (jj < stage_pieces) *reinterpret_cast<u32x4*>(dst + jj * 4096) = stage[jj];
       s_ascale[half * BM + 64 * q + lane] = stage_s;
-      // tile piece p = q + 4 jj: channel rows 16 (p / 2) + lane / 4, chunk 4 (p % 2) + lane % 4 of the
-      // row, in slot chunk ^ ((row >> 1) & 7); 16 (p / 2) does not change the key
-      const int r = lane >> 2, key = (lane >> 3) & 7;
+      // tile piece p = q + 4 jj: channel rows 16 (p / 2) + mx_tile_row(lane), chunk 4 (p % 2) +
+      // lane % 4 of the row, in slot chunk ^ ((row >> 1) & 7); 16 (p / 2) does not change the key
+      const int r = mx_tile_row(lane), key = (r >> 1) & 7;
       const int kc = 4 * (q & 1) + (lane & 3);  // p % 2 == q % 2
       uint8_t* wdst = smem_raw + half * UNIT_BYTES + A_BYTES + ((kc ^ key) << 4);
 #pragma unroll
