@@ -227,6 +227,95 @@ __global__ __launch_bounds__(256) void dispatch_index_kernel(
   perm[row] = t;
 }
 
+// dispatch_scan_kernel and dispatch_index_kernel in one launch, for up to kIndexScanBlocks counting
+// blocks: the table of per-block counts is a few KB in L2, so EVERY block of the index pass works the
+// scan out for itself in LDS (a microsecond, all blocks at once) instead of waiting for a launch of
+// one block to do it; block 0 writes counts and offsets for the kernels that follow.  block_counts
+// stays as the counting pass wrote it.  Same integers as the two kernels.
+constexpr int kIndexScanBlocks = 64;
+__global__ __launch_bounds__(256) void dispatch_index_scan_kernel(
+    const int32_t* __restrict__ topk_idx, int T, int K, int E, int tile_m, int64_t max_rows,
+    unsigned pair_blocks, const int32_t* __restrict__ block_counts, int num_blocks,
+    const int32_t* __restrict__ rank, int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
+    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm) {
+  extern __shared__ int32_t s_tab[];
+  int32_t* s_off = s_tab;           // [E + 1]
+  int32_t* s_cnt = s_off + E + 1;   // [E]
+  int32_t* s_pre = s_cnt + E;       // [2][E]: rows of the counting blocks before b0 and before b0 + 1
+  __shared__ int32_t s_wave_tot[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const bool pair_block = blockIdx.x < pair_blocks;
+  // the block's 256 pairs belong to at most 256 tokens, i.e. to counting blocks b0 and b0 + 1
+  const int b0 = pair_block ? (int)(((int64_t)blockIdx.x * 256 / K) / kDispTok) : 0;
+  int carried = 0;
+  for (int e0 = 0; e0 < E; e0 += 256) {
+    const int ex = e0 + tid, par = (e0 >> 8) & 1;
+    int padded = 0;
+    if (ex < E) {
+      int run = 0, pre0 = 0, pre1 = 0;
+      for (int i0 = 0; i0 < num_blocks; i0 += 16) {
+        int c[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          c[i] = block_counts[(size_t)(i0 + i < num_blocks ? i0 + i : 0) * E + ex];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          if (i0 + i == b0) pre0 = run;
+          if (i0 + i == b0 + 1) pre1 = run;
+          if (i0 + i < num_blocks) run += c[i];
+        }
+      }
+      s_cnt[ex] = run;
+      s_pre[ex] = pre0;
+      s_pre[E + ex] = pre1;
+      padded = (run + tile_m - 1) / tile_m * tile_m;
+    }
+    int incl = padded;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      int v = __shfl_up(incl, off, kWave);
+      if (lane >= off) incl += v;
+    }
+    if (lane == 63) s_wave_tot[par][wave] = incl;
+    __syncthreads();
+    int base = carried;
+    for (int w = 0; w < wave; ++w) base += s_wave_tot[par][w];
+    if (ex < E) s_off[ex] = base + incl - padded;
+    if (ex == E - 1) s_off[E] = base + incl;
+    for (int w = 0; w < 4; ++w) carried += s_wave_tot[par][w];
+  }
+  __syncthreads();
+  if (blockIdx.x == 0) {
+    for (int e = tid; e < E; e += 256) {
+      counts[e] = s_cnt[e];
+      offsets[e] = s_off[e];
+    }
+    if (tid == 0) offsets[E] = s_off[E];
+  }
+  if (!pair_block) {
+    const int idx = blockIdx.x - pair_blocks;
+    if (idx < E) {
+      const int64_t lo = (int64_t)s_off[idx] + s_cnt[idx], hi = s_off[idx + 1];
+      for (int64_t r = lo + tid; r < hi; r += 256) perm[r] = -1;
+    } else {
+      const int64_t r = (int64_t)s_off[E] + (int64_t)(idx - E) * 256 + tid;
+      if (r < max_rows) perm[r] = -1;
+    }
+    return;
+  }
+  const int64_t p = (int64_t)blockIdx.x * 256 + tid;
+  if (p >= (int64_t)T * K) return;
+  const int t = (int)(p / K);
+  const int e = topk_idx[p];
+  if (e < 0 || e >= E) {
+    inv_perm[p] = -1;
+    return;
+  }
+  const int row = s_off[e] + s_pre[(t / kDispTok - b0) * E + e] + rank[p];
+  inv_perm[p] = row;
+  perm[row] = t;
+}
+
 // All of dispatch for at most 256 tokens when no rows are copied (xe == NULL): count, scan and
 // index in one block.  A decode step spends more on starting three kernels than on their work.
 // Same arithmetic as the three kernels above, so the results are identical.
@@ -376,13 +465,21 @@ extern "C" int fs2moe_dispatch(const int32_t* topk_idx, const float* topk_w, con
                          topk_idx, T, K, E, block_counts, rank);
     if (int rc = check_launch("dispatch_count")) return rc;
   }
-  hipLaunchKernelGGL(dispatch_scan_kernel, dim3(1), dim3(256), 0, s, block_counts, nb, E, tile_m,
-                     counts, offsets);
-  if (int rc = check_launch("dispatch_scan")) return rc;
   // pair blocks, then E padding blocks, then blocks for the rows beyond offsets[E] (at most
   // max_rows - T*K of them, since offsets[E] >= T*K)
   const int64_t pairs = (int64_t)T * K;
   const unsigned tail_blocks = (unsigned)((max_rows - pairs + 255) / 256);
+  if (xe == nullptr && nb <= kIndexScanBlocks) {
+    const unsigned pair_blocks = (unsigned)((pairs + 255) / 256);
+    const size_t lds = (size_t)(4 * E + 1) * sizeof(int32_t);
+    hipLaunchKernelGGL(dispatch_index_scan_kernel, dim3(pair_blocks + (unsigned)E + tail_blocks),
+                       dim3(256), lds, s, topk_idx, T, K, E, tile_m, max_rows, pair_blocks,
+                       block_counts, nb, rank, counts, offsets, perm, inv_perm);
+    return check_launch("dispatch_index_scan");
+  }
+  hipLaunchKernelGGL(dispatch_scan_kernel, dim3(1), dim3(256), 0, s, block_counts, nb, E, tile_m,
+                     counts, offsets);
+  if (int rc = check_launch("dispatch_scan")) return rc;
   if (xe == nullptr) {
     const unsigned pair_blocks = (unsigned)((pairs + 255) / 256);
     hipLaunchKernelGGL(dispatch_index_kernel, dim3(pair_blocks + (unsigned)E + tail_blocks),

@@ -244,9 +244,12 @@ def test_dispatch_matches_oracle(gpu_device, dtype, tile_m, scale_input):
     assert torch.equal(xe, want)
 
 
-@pytest.mark.parametrize("tokens,e,k", [(1, 8, 2), (200, 256, 16), (256, 128, 8), (257, 128, 8), (700, 24, 4)])
+@pytest.mark.parametrize("tokens,e,k", [(1, 8, 2), (200, 256, 16), (256, 128, 8), (257, 128, 8), (700, 24, 4),
+                                        (5000, 40, 3), (1100, 384, 24), (16384, 8, 1), (16500, 16, 2)])
 def test_dispatch_without_row_copy_matches_oracle(gpu_device, tokens, e, k):
-    # at most 256 tokens take the one-kernel path, more the three-kernel path: same artefacts
+    # at most 256 tokens take the one-kernel path; up to 64 counting blocks (16384 tokens) two kernels,
+    # the second doing the scan in every block (with top-3 its blocks of 256 pairs straddle counting
+    # blocks); more the three-kernel path: same artefacts
     _say("dispatch index only", tokens, e, k)
     spec = W.small_spec(tokens=tokens, model_dim=64, num_experts=e, top_k=k, inner_dim=8, dtype="bf16",
                         zipf_s=1.1, seed=tokens + e)
