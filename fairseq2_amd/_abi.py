@@ -15,10 +15,11 @@ from torch import Tensor
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfs2moe.so")
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
+ROUTER_OUT_IN = 0x100  # OR-ed into score_fn: the router argument is (E, D)
 W_IN_OUT, W_OUT_IN = 0, 1
 MAX_EXPERTS, MAX_TOP_K = 512, 32
 
@@ -27,6 +28,7 @@ _PROTOTYPES = {
     "fs2moe_abi_version": (c_int32, []),
     "fs2moe_last_error": (c_char_p, []),
     "fs2moe_router_workspace_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32]),
+    "fs2moe_router_takes_out_in": (c_int32, [c_int32, c_int32, c_int32, c_int32]),
     "fs2moe_router_topk": (
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
@@ -242,8 +244,10 @@ def router_topk(
     renormalize: bool = False,
     want_logits: bool = False,
     split: bool = True,
+    router_t: Tensor | None = None,
 ) -> tuple[Tensor, Tensor, Tensor | None]:
     """``x`` (T, D), ``router`` (D, E) -> ``topk_idx`` int32 (T, K), ``topk_w`` f32 (T, K), logits.
+    ``router_t``: optionally the same matrix expert-major, (E, D), used where the library reads it.
 
     ``split=False`` withholds the scratch buffer that lets several blocks share a token tile when
     there are few tokens (see ``fs2moe_router_topk``)."""
@@ -257,8 +261,9 @@ def router_topk(
     logits = torch.empty((t, e), dtype=torch.float32, device=x.device) if want_logits else None
     if bias is not None and (bias.dtype != torch.float32 or bias.numel() != e):
         raise ValueError("router bias must be f32 of E elements")
+    mat, score_fn = router_operand(lib, x, router, router_t, score_fn)
     rc = lib.fs2moe_router_topk(
-        _ptr(x), _ptr(router), _ptr(bias), t, d, e, top_k, dtype_code(x.dtype), score_fn,
+        _ptr(x), _ptr(mat), _ptr(bias), t, d, e, top_k, dtype_code(x.dtype), score_fn,
         int(renormalize), _ptr(idx), _ptr(w), _ptr(logits), *_router_workspace(lib, x, e, split), _stream(),
     )
     _check(rc, "fs2moe_router_topk")
@@ -278,6 +283,41 @@ def cpu_router_select(logits: Tensor, top_k: int, score_fn: int = SCORE_SIGMOID,
                                       idx.data_ptr(), w.data_ptr())
     _check(rc, "fs2moe_cpu_router_select")
     return idx, w
+
+
+def router_expert_major(router: Tensor, holder=None) -> Tensor | None:
+    """The bf16 router matrix expert-major, ``(E, D)``: a derived copy that the router kernel reads
+    without transposing (``ROUTER_OUT_IN``).  It is kept on ``holder`` (the module that owns the
+    parameter; by default the tensor object itself, which for a parameter lives as long as its
+    module) and made again whenever the parameter has changed: in-place updates bump its version
+    counter, a move or a new tensor changes its address.  None for other dtypes."""
+    if router.dtype != torch.bfloat16 or not router.is_cuda:
+        return None
+    holder = router if holder is None else holder
+    key = (router._version, router.data_ptr(), tuple(router.shape))
+    hit = getattr(holder, "_fs2moe_router_t", None)
+    if hit is None or hit[0] != key:
+        with torch.no_grad():
+            hit = (key, router.detach().t().contiguous())
+        try:
+            object.__setattr__(holder, "_fs2moe_router_t", hit)
+        except (AttributeError, TypeError):
+            pass  # nowhere to keep it: made again on the next call
+    return hit[1]
+
+
+def router_operand(lib, x: Tensor, router: Tensor, router_t: Tensor | None, score_fn: int) -> tuple[Tensor, int]:
+    """The router matrix to pass and the score_fn to pass with it: the expert-major copy ``router_t``
+    ``(E, D)`` with ``ROUTER_OUT_IN`` set where the library reads that form at this size, else
+    ``router`` ``(D, E)``."""
+    if router_t is None:
+        return router, score_fn
+    d, e = router.shape
+    if router_t.shape != (e, d) or router_t.dtype != router.dtype or not router_t.is_contiguous():
+        raise ValueError("router_t must be the contiguous (E, D) transpose of router")
+    if lib.fs2moe_router_takes_out_in(x.shape[0], d, e, dtype_code(x.dtype)):
+        return router_t, score_fn | ROUTER_OUT_IN
+    return router, score_fn
 
 
 def _router_workspace(lib, x: Tensor, num_experts: int, split: bool) -> tuple[int | None, int]:
@@ -305,6 +345,7 @@ def router_topk_norm(
     renormalize: bool = False,
     want_logits: bool = False,
     split: bool = True,
+    router_t: Tensor | None = None,
 ) -> tuple[Tensor, Tensor, Tensor, Tensor | None]:
     """RMS-normalises the rows of ``x`` and routes the result: ``xn``, then as :func:`router_topk`."""
     lib = load()
@@ -319,8 +360,9 @@ def router_topk_norm(
     idx = torch.empty((t, top_k), dtype=torch.int32, device=x.device)
     w = torch.empty((t, top_k), dtype=torch.float32, device=x.device)
     logits = torch.empty((t, e), dtype=torch.float32, device=x.device) if want_logits else None
+    mat, score_fn = router_operand(lib, x, router, router_t, score_fn)
     rc = lib.fs2moe_router_topk_norm(
-        _ptr(x), _ptr(norm_weight), float(norm_eps), _ptr(xn), _ptr(router), _ptr(bias), t, d, e,
+        _ptr(x), _ptr(norm_weight), float(norm_eps), _ptr(xn), _ptr(mat), _ptr(bias), t, d, e,
         top_k, dtype_code(x.dtype), score_fn, int(renormalize), _ptr(idx), _ptr(w), _ptr(logits),
         *_router_workspace(lib, x, e, split), _stream(),
     )
@@ -928,8 +970,10 @@ def forward(
     workspace: Tensor | None = None,
     residual: Tensor | None = None,
     norm: tuple[Tensor | None, float] | None = None,
+    router_t: Tensor | None = None,
 ) -> Tensor:
     """The whole layer through ``fs2moe_forward``: one call, intermediates in one workspace.
+    ``router_t``: optionally the router matrix expert-major, (E, D), used where the library reads it.
     With ``residual`` ``(T, D)`` the result is ``residual + layer(x)`` from the same accumulation.
     With ``norm`` = (weight or None, eps) the rows are RMS-normalised on the way into the router
     (``fs2moe_forward_norm``): the result is ``[residual +] layer(rms_norm(x))``.
@@ -956,8 +1000,9 @@ def forward(
     out = torch.empty_like(x)
     sg, su, sd = scales if scales is not None else (None, None, None)
     hg, hu, hd = shared if shared is not None else (None, None, None)
+    mat, score_fn = router_operand(lib, x, router, router_t, score_fn)
     tail = (
-        _ptr(residual), _ptr(router), _ptr(router_bias), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(sg),
+        _ptr(residual), _ptr(mat), _ptr(router_bias), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(sg),
         _ptr(su), _ptr(sd), _ptr(hg), _ptr(hu), _ptr(hd), t, d, num_experts, top_k, f, f_shared,
         tile_m, dtype_code(x.dtype), dtype_code(w_gate.dtype), score_fn, int(renormalize),
         int(scale_input), _ptr(workspace), workspace.numel(), _ptr(out), _stream(),

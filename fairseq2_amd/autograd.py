@@ -127,9 +127,10 @@ def forward_saving(x, residual, router, wg, wu, wd, sg, su, sd, cfg, norm_w=None
     score_fn, renorm, scale_input = cfg["score_fn"], cfg["renormalize"], cfg["scale_input"]
     if cfg.get("norm_eps") is not None:
         x, idx, w, logits = _abi.router_topk_norm(x, norm_w, cfg["norm_eps"], router, cfg["router_bias"], k,
-                                                  score_fn, renorm, want_logits=True)
+                                                  score_fn, renorm, want_logits=True, router_t=cfg.get("router_t"))
     else:
-        idx, w, logits = _abi.router_topk(x, router, cfg["router_bias"], k, score_fn, renorm, want_logits=True)
+        idx, w, logits = _abi.router_topk(x, router, cfg["router_bias"], k, score_fn, renorm, want_logits=True,
+                                          router_t=cfg.get("router_t"))
     disp = _abi.dispatch(idx, w, x, e, tile_m, scale_input, gather=True)
     ye, g, u = experts_forward(disp.xe, disp.counts, disp.offsets, wg, wu, wd, e, cfg.get("activation"),
                                rows_per_expert=x.shape[0] if x.shape[0] <= 16 else 0)

@@ -570,6 +570,183 @@ __global__ __launch_bounds__(rmfma::Shape<NF>::THREADS) void router_mfma_kernel(
   }
 }
 
+// ------------------------------------------------------------------ bf16 / MFMA, (E, D) router matrix
+// The same 32-token block with the router matrix given expert-major ((E, D): each expert's weights
+// contiguous, e.g. a transposed copy the caller keeps).  Then both MFMA operands are k-contiguous:
+// token rows and expert rows travel global -> LDS as 128-byte row pieces by direct loads
+// (buffer_load ... lds: no staging registers, no LDS store instructions) and come back as plain
+// 16-byte fragment reads, where the (D, E) form stores 20 KB per step to LDS and reads the matrix
+// back through transposing reads at a quarter of the rate.  A tile is 64 of k: 32 token rows + EP
+// expert rows; a step is TPS tiles, SLOTS steps in a ring, SLOTS - 1 of them in flight.  Wave w
+// multiplies a tile's 16-k slice w / 4 into expert fragment w % 4 (+ 4, ..); the four slices' sums meet in
+// LDS and are added in a fixed order, then every wave selects for two tokens, as above.
+// Row r of a tile is 128 bytes; its 16-byte chunk c sits in slot c ^ ((r >> 1) & 7) (chosen by which
+// chunk a lane fetches: the direct loads put lane l's 16 bytes at l * 16 of the piece), so the
+// fragment reads of 32 rows are free of bank conflicts.
+namespace rmfma_t {
+constexpr int BT = 32, BK = 64;
+template <int NF>
+struct Shape {
+  static constexpr int EP = 128 * NF;
+  static constexpr int TILE_BYTES = (BT + EP) * BK * 2;  // token rows first, then expert rows
+  // tiles per step, i.e. per barrier: two where the ring then still holds three steps (one tile per
+  // step and seven in the ring: 18.3 us for 8192 tokens of 2048 features against 15.9 this way;
+  // the transposing kernel above 19.7)
+  static constexpr int TPS = NF == 1 ? 2 : 1;
+  static constexpr int STEP_BYTES = TPS * TILE_BYTES;
+  static constexpr int SLOTS = (148 * 1024) / STEP_BYTES;
+  static constexpr int LDL = EP + 4;                     // logits row stride (floats)
+  static constexpr int LOGIT_BYTES = 4 * BT * LDL * 4;   // the four slices' partial sums
+  static constexpr int RING_BYTES = SLOTS * STEP_BYTES;
+  static constexpr int SMEM_BYTES = RING_BYTES > LOGIT_BYTES ? RING_BYTES : LOGIT_BYTES;
+};
+}  // namespace rmfma_t
+
+template <int NF>
+__global__ __launch_bounds__(1024) void router_mfma_t_kernel(
+    const uint16_t* x, const uint16_t* norm_w, float norm_eps, uint16_t* xn,
+    const uint16_t* __restrict__ router_t, const float* __restrict__ bias, int T, int D, int E, int K,
+    int score_fn, int renorm, int32_t* __restrict__ topk_idx, float* __restrict__ topk_w,
+    float* __restrict__ logits) {
+  using namespace rmfma_t;
+  using S = Shape<NF>;
+  constexpr int EP = S::EP, LDL = S::LDL, SLOTS = S::SLOTS, AHEAD = SLOTS - 1, J = EP / 64, TPS = S::TPS;
+  static_assert(AHEAD >= 1 && (AHEAD - 1) * TPS * (NF + 1) < 64, "ring and wait counts");
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_t[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // 0 .. 15
+  const int lr = lane & 31, lk = lane >> 5;
+  const int t0 = blockIdx.x * BT;
+  if (xn != nullptr) {
+    rms_norm_block_rows<uint16_t>(x, norm_w, norm_eps, xn, t0, T - t0 < BT ? T - t0 : BT, D, 0, D);
+    __syncthreads();  // the block's rows of xn are written and visible to all its waves
+    x = xn;
+  }
+  float b[J];
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    const int e = lane + 64 * j;
+    b[j] = (bias != nullptr && e < E) ? bias[e] : 0.f;
+  }
+
+  // ---- what this wave loads per step: expert pieces wave + 16 j (8 rows x 128 bytes each), and
+  // waves 0..3 token piece `wave`.  Lane l fills row l / 8, slot l % 8 of its piece.
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(x + (size_t)t0 * D), 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t r_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(router_t), 0, -1, 0x00020000);
+  const int prow = lane >> 3, pslot = lane & 7;
+  // (off_r has a size that does not depend on NF on purpose: with a template-dependent argument the
+  // host pass cannot check the call of the load builtin below, drops the kernel's instantiation
+  // without a message, and the library ends up with an undefined kernel symbol)
+  uint32_t off_r[2] = {0u, 0u}, off_x = 0;
+  static_assert(NF <= 2, "off_r");
+#pragma unroll
+  for (int j = 0; j < NF; ++j) {
+    const int row = 8 * (wave + 16 * j) + prow;  // expert
+    const int kc = pslot ^ ((row >> 1) & 7);
+    const int e = row < E ? row : E - 1;          // (logits of experts past E are never looked at)
+    off_r[j] = (uint32_t)(((size_t)e * D + kc * 8) * 2);
+  }
+  const bool loads_x = wave < BT / 8;
+  if (loads_x) {
+    const int row = 8 * wave + prow;  // token of the tile
+    const int kc = pslot ^ ((row >> 1) & 7);
+    const int t = t0 + row < T ? row : T - 1 - t0;  // (rows past T are never looked at)
+    off_x = (uint32_t)(((size_t)t * D + kc * 8) * 2);
+  }
+  const int steps = D / (BK * TPS);  // the host sends only D % (64 TPS) == 0 here
+  auto issue = [&](int step) {
+    uint8_t* slot = smem_t + (step % SLOTS) * S::STEP_BYTES;
+#pragma unroll
+    for (int tt = 0; tt < TPS; ++tt) {
+      uint8_t* tile = slot + tt * S::TILE_BYTES;
+      const uint32_t koff = (uint32_t)(step * TPS + tt) * (BK * 2);
+      if (loads_x)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (lds_ptr)(tile + wave * 1024), 16, off_x, koff, 0, 0);
+#pragma unroll
+      for (int j = 0; j < NF; ++j)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            r_rsrc, (lds_ptr)(tile + BT * BK * 2 + (wave + 16 * j) * 1024), 16, off_r[j], koff, 0, 0);
+    }
+  };
+
+  f32x16 acc[NF];
+#pragma unroll
+  for (int f = 0; f < NF; ++f)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[f][i] = 0.f;
+  // fragment addresses within a tile: token row lr / expert row 32 F + lr, chunk 2 ks + lk (the key
+  // is (lr >> 1) & 7 for all of them: 32 F does not change it)
+  const int ks = wave >> 2, f0 = wave & 3;
+  const uint32_t frag = (uint32_t)(lr * 128 + (((2 * ks + lk) ^ ((lr >> 1) & 7)) << 4));
+
+  for (int st = 0; st < AHEAD && st < steps; ++st) issue(st);
+  for (int st = 0; st < steps; ++st) {
+    // this wave's loads of step st have landed once at most the loads of the AHEAD - 1 steps issued
+    // after them are outstanding (vmcnt counts in issue order); towards the end fewer steps follow
+    if (st + AHEAD - 1 < steps) {
+      constexpr int R_ONLY = (AHEAD - 1) * TPS * NF, WITH_X = (AHEAD - 1) * TPS * (NF + 1);
+      if (loads_x) __builtin_amdgcn_s_waitcnt(0x0f70 | (WITH_X & 15) | ((WITH_X >> 4) << 14));
+      else __builtin_amdgcn_s_waitcnt(0x0f70 | (R_ONLY & 15) | ((R_ONLY >> 4) << 14));
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    }
+    lds_barrier();  // every wave's part of step st is in LDS; everybody is done with step st - 1
+    if (st + AHEAD < steps) issue(st + AHEAD);  // into the slot of step st - 1
+    const uint8_t* slot = smem_t + (st % SLOTS) * S::STEP_BYTES;
+    bf16x8 xf[TPS], rf[TPS][NF];
+#pragma unroll
+    for (int tt = 0; tt < TPS; ++tt) {
+      const uint8_t* tile = slot + tt * S::TILE_BYTES;
+      xf[tt] = lds_read_frag(reinterpret_cast<const uint16_t*>(tile + frag));
+#pragma unroll
+      for (int f = 0; f < NF; ++f)
+        rf[tt][f] = lds_read_frag(
+            reinterpret_cast<const uint16_t*>(tile + BT * BK * 2 + (f0 + 4 * f) * 32 * 128 + frag));
+    }
+#pragma unroll
+    for (int tt = 0; tt < TPS; ++tt)
+#pragma unroll
+      for (int f = 0; f < NF; ++f)
+        acc[f] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rf[tt][f], xf[tt], acc[f], 0, 0, 0);
+  }
+  __syncthreads();  // all fragment reads done: the ring becomes the partial sums' space
+
+  // Partial logits of slice ks -> its LDS region.  Accumulator layout: lane holds token lr and
+  // experts 32 F + 8 q + 4 lk + j (F = f0 + 4 f).
+  float* sL = reinterpret_cast<float*>(smem_t) + ks * (BT * LDL);
+#pragma unroll
+  for (int f = 0; f < NF; ++f)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e = (f0 + 4 * f) * 32 + 8 * q + 4 * lk;
+      f32x4 v = {acc[f][4 * q], acc[f][4 * q + 1], acc[f][4 * q + 2], acc[f][4 * q + 3]};
+      *reinterpret_cast<f32x4*>(&sL[lr * LDL + e]) = v;
+    }
+  __syncthreads();
+
+  constexpr int TPW = BT / 16;  // every wave selects for two tokens
+  for (int i = 0; i < TPW; ++i) {
+    const int tl = wave * TPW + i;
+    const int t = t0 + tl;
+    if (t >= T) break;  // wave-uniform
+    float v[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+      const int e = lane + 64 * j;
+      float sum = 0.f;
+#pragma unroll
+      for (int g2 = 0; g2 < 4; ++g2) sum += reinterpret_cast<const float*>(smem_t)[g2 * (BT * LDL) + tl * LDL + e];
+      v[j] = sum + b[j];
+      if (logits != nullptr && e < E) logits[(size_t)t * E + e] = v[j];
+    }
+    select_topk<J>(v, lane, t, E, K, score_fn, renorm, topk_idx, topk_w);
+  }
+}
+
 constexpr int kMaxSlices = 8;  // blocks sharing a token tile, at most
 
 // Second half of the split router: one wave per token adds the `slices` partial logits in
@@ -883,6 +1060,15 @@ static int router_slices(int T, int D, int E, int act_dtype) {
   return s >= 2 ? s : 1;
 }
 
+// Whether the router of this size reads an (E, D) matrix (FS2MOE_ROUTER_OUT_IN): the bf16 MFMA path
+// with one block per token tile and whole steps of k.  Where several blocks would share a token tile
+// (few tokens) the split kernels above are faster (64 tokens of 2048 features: 6.6 + 5.6 us against
+// 16.9 us), and they read (D, E).
+static bool router_takes_out_in(int T, int D, int E, int act_dtype) {
+  return act_dtype == FS2MOE_BF16 && D % (rmfma_t::BK * 2) == 0 && E % 8 == 0 && E <= 256 && T > rmfma::BT &&
+         (int64_t)E * D * 2 < (1ll << 31) && D <= (1 << 20) && router_slices(T, D, E, act_dtype) == 1;
+}
+
 extern "C" int64_t fs2moe_router_workspace_bytes(int32_t T, int32_t D, int32_t E,
                                                  int32_t act_dtype) {
   if (T < 0 || D < 1 || E < 1) return -1;
@@ -904,10 +1090,16 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
               FS2MOE_MAX_EXPERTS);
   FS2_REQUIRE(K >= 1 && K <= E && K <= FS2MOE_MAX_TOP_K, "router: K=%d outside [1, min(E=%d, %d)]",
               K, E, FS2MOE_MAX_TOP_K);
+  const bool out_in = (score_fn & FS2MOE_ROUTER_OUT_IN) != 0;
+  score_fn &= ~FS2MOE_ROUTER_OUT_IN;
   FS2_REQUIRE(score_fn == FS2MOE_SCORE_SIGMOID || score_fn == FS2MOE_SCORE_SOFTMAX,
               "router: unknown score_fn %d", score_fn);
   FS2_REQUIRE(act_dtype == FS2MOE_F32 || act_dtype == FS2MOE_BF16, "router: act_dtype %d",
               act_dtype);
+  FS2_REQUIRE(!out_in || (router_takes_out_in(T, D, E, act_dtype) && aligned16(x) && aligned16(router) &&
+                          aligned16(xn)),
+              "router: an (E, D) router matrix is read only where fs2moe_router_takes_out_in says so "
+              "(T=%d D=%d E=%d), from 16-byte aligned operands", T, D, E);
   if (T == 0) return FS2MOE_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   // (a single token tile of the bf16 MFMA router normalises in its own blocks, also when several
@@ -928,6 +1120,37 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
     x = xn;
     xn = nullptr;
     norm_w = nullptr;
+  }
+  if (out_in) {
+    auto k1 = router_mfma_t_kernel<1>;
+    auto k2 = router_mfma_t_kernel<2>;
+    static bool attr_set = false;  // benign race: setting the attribute is idempotent
+    if (!attr_set) {
+      hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(k1),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          rmfma_t::Shape<1>::SMEM_BYTES);
+      hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(k2),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          rmfma_t::Shape<2>::SMEM_BYTES);
+      if (e1 != hipSuccess || e2 != hipSuccess) {
+        set_error("router: cannot reserve LDS: %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+        return FS2MOE_ERR_LAUNCH;
+      }
+      attr_set = true;
+    }
+    const dim3 grid((T + rmfma_t::BT - 1) / rmfma_t::BT), threads(1024);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    const uint16_t* wp = static_cast<const uint16_t*>(norm_w);
+    uint16_t* xnp = static_cast<uint16_t*>(xn);
+    if (E <= 128)
+      hipLaunchKernelGGL(k1, grid, threads, rmfma_t::Shape<1>::SMEM_BYTES, s, xp, wp, norm_eps, xnp,
+                         static_cast<const uint16_t*>(router), bias, T, D, E, K, score_fn, renormalize,
+                         topk_idx, topk_w, logits);
+    else
+      hipLaunchKernelGGL(k2, grid, threads, rmfma_t::Shape<2>::SMEM_BYTES, s, xp, wp, norm_eps, xnp,
+                         static_cast<const uint16_t*>(router), bias, T, D, E, K, score_fn, renormalize,
+                         topk_idx, topk_w, logits);
+    return check_launch("router_mfma (E, D)");
   }
   if (act_dtype == FS2MOE_F32) {
     // The MFMA path moves 16-byte chunks (D and E multiples of 4, aligned bases) and holds up to
@@ -1032,6 +1255,10 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
   }
   return launch_router_fma<uint16_t>(x, norm_w, norm_eps, xn, router, bias, T, D, E, K, score_fn, renormalize, topk_idx,
                                      topk_w, logits, s);
+}
+
+extern "C" int32_t fs2moe_router_takes_out_in(int32_t T, int32_t D, int32_t E, int32_t act_dtype) {
+  return router_takes_out_in(T, D, E, act_dtype) ? 1 : 0;
 }
 
 extern "C" int fs2moe_router_topk(const void* x, const void* router, const float* bias, int32_t T,

@@ -579,6 +579,8 @@ class MoE(FeedForwardNetwork):
             scale_input=self.scale_on == "input", router_bias=self.router_bias,
             activation=None if ex.has_fused_gate else ex.activation,
             norm_eps=None if norm_args is None else norm_args[1],
+            # the forward pass routes as the inference path does (the same logits bit for bit)
+            router_t=self._router_expert_major(),
         )
         out = MoEFunction.apply(x, res, self.router, ex.gate_proj, ex.inner_proj, ex.output_proj,
                                 *shared, None if norm_args is None else norm_args[0], cfg)
@@ -612,6 +614,10 @@ class MoE(FeedForwardNetwork):
             weight = (weight if allow_grad else weight.detach()).contiguous()
         return weight, float(norm.eps)
 
+    def _router_expert_major(self) -> Tensor | None:
+        """The router matrix expert-major (see :func:`fairseq2_amd._abi.router_expert_major`)."""
+        return _abi.router_expert_major(self.router, self)
+
     def _single_call(self, x: Tensor, residual: Tensor | None = None, norm=None) -> Tensor:
         """The layer through the library's whole-layer entry point: one call, one workspace
         allocation (same kernels and results as :meth:`_stages`)."""
@@ -644,7 +650,7 @@ class MoE(FeedForwardNetwork):
             x, self.router.detach(), self.router_bias, *weights, ex.num_local_experts, self.top_k,
             scales=scales, shared=shared, tile_m=self.tile_m, score_fn=_SCORE_FNS[self.score_fn],
             renormalize=self.renormalize, scale_input=self.scale_on == "input", residual=residual,
-            norm=norm,
+            norm=norm, router_t=self._router_expert_major(),
         )
 
     @torch.no_grad()
@@ -653,13 +659,13 @@ class MoE(FeedForwardNetwork):
         if norm is None:
             idx, w, _ = _abi.router_topk(
                 x, self.router.detach(), self.router_bias, self.top_k, _SCORE_FNS[self.score_fn],
-                self.renormalize,
+                self.renormalize, router_t=self._router_expert_major(),
             )
         else:
             # every later stage reads the normalised rows
             x, idx, w, _ = _abi.router_topk_norm(
                 x, norm[0], norm[1], self.router.detach(), self.router_bias, self.top_k,
-                _SCORE_FNS[self.score_fn], self.renormalize,
+                _SCORE_FNS[self.score_fn], self.renormalize, router_t=self._router_expert_major(),
             )
         scale_input = self.scale_on == "input"
         # Unscaled rows need no copy in expert order: the first GEMM reads them from x through the

@@ -57,6 +57,7 @@ def moe_forward(
         shared=None if shared_gate is None else (shared_gate, shared_up, shared_down),
         tile_m=tile_m, score_fn=score_fn, renormalize=renormalize, scale_input=scale_input,
         residual=residual, norm=(norm_weight, norm_eps) if normed else None,
+        router_t=_abi.router_expert_major(router),
     )
 
 
@@ -93,7 +94,7 @@ def moe_backward(
 
     cfg = dict(num_experts=num_experts, top_k=top_k, tile_m=tile_m, score_fn=score_fn,
                renormalize=renormalize, scale_input=scale_input, router_bias=router_bias,
-               norm_eps=norm_eps if normed else None)
+               norm_eps=norm_eps if normed else None, router_t=_abi.router_expert_major(router))
     _, saved = forward_saving(x, None, router, w_gate, w_up, w_down, shared_gate, shared_up,
                               shared_down, cfg, norm_weight)
     grads = list(backward_from(saved[12] if normed else x, router, w_gate, w_up, w_down, shared_gate,

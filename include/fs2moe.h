@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FS2MOE_ABI_VERSION 13
+#define FS2MOE_ABI_VERSION 14
 
 /* element types */
 #define FS2MOE_F32 0
@@ -36,6 +36,11 @@ extern "C" {
 /* router score functions */
 #define FS2MOE_SCORE_SIGMOID 0 /* reference: sigmoid of the selected raw logit (moe.py:113,127) */
 #define FS2MOE_SCORE_SOFTMAX 1 /* extension: softmax over all experts */
+/* May be OR-ed into a score_fn argument: `router` then points at an (E, D) matrix (each expert's
+ * weights contiguous: the transpose of the reference's parameter, e.g. a copy the caller keeps and
+ * refreshes when the parameter changes) instead of (D, E).  Read that way the router's bf16 kernel
+ * needs no transposing reads.  Accepted only where fs2moe_router_takes_out_in returns 1. */
+#define FS2MOE_ROUTER_OUT_IN 0x100
 
 /* weight orientation of a GLU network */
 #define FS2MOE_W_IN_OUT 0 /* (E*in, out), out contiguous: grouped experts (experts.py:53-82) */
@@ -76,6 +81,11 @@ const char* fs2moe_last_error(void);
  *   summation order only.
  */
 int64_t fs2moe_router_workspace_bytes(int32_t T, int32_t D, int32_t E, int32_t act_dtype);
+/* 1 if the router of this size reads an (E, D) matrix when FS2MOE_ROUTER_OUT_IN is set (bf16, D a
+ * multiple of 128, E a multiple of 8 up to 256, enough tokens that every token tile of 32 has a block
+ * of its own: more than 4096, or a narrow model), else 0: then pass (D, E).
+ * No counterpart in the reference (its router parameter is (D, E): llama4/moe.py:75-77). */
+int32_t fs2moe_router_takes_out_in(int32_t T, int32_t D, int32_t E, int32_t act_dtype);
 int fs2moe_router_topk(const void* x, const void* router, const float* bias, int32_t T, int32_t D,
                        int32_t E, int32_t K, int32_t act_dtype, int32_t score_fn,
                        int32_t renormalize, int32_t* topk_idx, float* topk_w, float* logits,

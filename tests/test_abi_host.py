@@ -40,7 +40,7 @@ def test_library_exports_every_declared_symbol(lib):
 
 
 def test_abi_version_and_limits(lib):
-    assert lib.fs2moe_abi_version() == _abi.ABI_VERSION == 13
+    assert lib.fs2moe_abi_version() == _abi.ABI_VERSION == 14
     assert re.search(rf"#define FS2MOE_ABI_VERSION {_abi.ABI_VERSION}\b", open(HEADER).read())
     text = open(HEADER).read()
     assert f"#define FS2MOE_MAX_EXPERTS {_abi.MAX_EXPERTS}" in text

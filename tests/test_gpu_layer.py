@@ -378,9 +378,42 @@ def test_single_call_entry_point_equals_the_module(gpu_device, dtype, weight_dty
     got = _abi.forward(
         x2, m.router.detach(), m.router_bias, *weights, 8, 2, scales=scales, shared=sh, tile_m=16,
         score_fn=_SCORE_FNS[mode.score_fn], renormalize=mode.renormalize, scale_input=mode.scale_on == "input",
+        router_t=m.router.detach().t().contiguous(),  # as the module passes it
     )
     torch.cuda.synchronize()
     assert torch.equal(got, out.reshape(-1, 128))
+
+
+def test_expert_major_copy_of_the_router_follows_the_parameter(gpu_device):
+    """The derived (E, D) copy the bf16 router reads: made once, made again after an in-place update,
+    after a move and for another tensor (also one that reuses a freed tensor's address), and kept
+    with its owner, not under an address."""
+    from fairseq2_amd import _abi
+
+    _say("router copy")
+    spec = W.small_spec(tokens=100, model_dim=128, num_experts=8, top_k=2, inner_dim=64, dtype="bf16", seed=3)
+    m = build_module(W.make_workload_from_spec(spec), gpu_device)
+    first = m._router_expert_major()
+    assert first.shape == (8, 128) and torch.equal(first, m.router.detach().t())
+    assert m._router_expert_major() is first, "kept between calls"
+    x = torch.randn(100, 128, generator=torch.Generator().manual_seed(1)).bfloat16().to(gpu_device)
+    with torch.no_grad():
+        before = m(x)
+        m.router.mul_(-1.0)  # an optimizer step's kind of update
+        second = m._router_expert_major()
+        assert second is not first and torch.equal(second, m.router.detach().t())
+        after = m(x)
+        idx_now = _abi.router_topk(x, m.router.detach(), m.router_bias, 2, router_t=second)[0]
+        idx_plain = _abi.router_topk(x, m.router.detach(), m.router_bias, 2)[0]
+    assert torch.equal(idx_now, idx_plain) and not torch.equal(before, after)
+    # tensors that come and go at one address: each gets its own copy
+    seen = set()
+    for i in range(4):
+        r = torch.full((128, 8), float(i), dtype=torch.bfloat16, device=gpu_device)
+        seen.add(r.data_ptr())
+        assert float(_abi.router_expert_major(r)[0, 0]) == float(i)
+        del r
+    assert _abi.router_expert_major(torch.zeros(4, 4, device=gpu_device)) is None, "f32: no copy"
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])

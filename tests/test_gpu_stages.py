@@ -171,6 +171,83 @@ def test_router_with_norm_in_front(gpu_device, dtype, tokens, d, e, k, with_weig
     assert torch.equal(idx, idx2) and torch.equal(w, w2) and torch.equal(logits, logits2)
 
 
+@pytest.mark.parametrize(
+    "tokens,d,e,k,mode,zipf",
+    [
+        (8192, 2048, 128, 8, "softmax_renorm", 1.2),  # the benchmark's layer
+        (33, 128, 8, 2, "reference", None),           # one step, a last block of one token
+        (4100, 256, 16, 4, "softmax_plain", None),
+        (4200, 1024, 256, 16, "sigmoid_renorm", 1.0),  # two expert fragments per wave
+        (4130, 384, 136, 3, "softmax_renorm", None),   # experts off the fragment size
+        (5000, 5120, 16, 1, "reference", None),
+    ],
+)
+def test_router_reading_an_expert_major_matrix(gpu_device, tokens, d, e, k, mode, zipf):
+    """The router given its matrix as (E, D) (ROUTER_OUT_IN): the same selection as the oracle's,
+    logits equal up to summation order, with exact ties, and with the
+    normalisation in front bit for bit what the plain call makes of the normalised rows."""
+    _say("router (E, D)", tokens, d, e, k, mode)
+    lib = _abi.load()
+    assert lib.fs2moe_router_takes_out_in(tokens, d, e, _abi.dtype_code(torch.bfloat16)) == 1
+    assert lib.fs2moe_router_takes_out_in(tokens, d, e, _abi.dtype_code(torch.float32)) == 0
+    assert lib.fs2moe_router_takes_out_in(32, d, e, _abi.dtype_code(torch.bfloat16)) == 0
+    # few tokens of a wide model: several blocks share a token tile, and those kernels read (D, E)
+    assert lib.fs2moe_router_takes_out_in(64, 2048, 128, _abi.dtype_code(torch.bfloat16)) == 0
+    assert lib.fs2moe_router_takes_out_in(tokens, d + 8, e, _abi.dtype_code(torch.bfloat16)) == 0
+    spec = W.small_spec(tokens=tokens, model_dim=d, num_experts=e, top_k=k, inner_dim=8, dtype="bf16",
+                        zipf_s=zipf, mode=MODES[mode], seed=tokens + e)
+    wl = W.make_workload_from_spec(spec, with_weights=False)
+    logits, idx, w = oracle_routing(wl)
+    x = wl.x.reshape(-1, d).bfloat16().to(gpu_device)
+    router = wl.router.bfloat16().to(gpu_device)
+    router_t = router.t().contiguous()
+    bias = None if wl.router_bias is None else wl.router_bias.to(gpu_device)
+    score = _abi.SCORE_SOFTMAX if "softmax" in mode else _abi.SCORE_SIGMOID
+    gi, gw, gl = _abi.router_topk(x, router, bias, k, score, spec.mode.renormalize, want_logits=True,
+                                  router_t=router_t)
+    np.testing.assert_allclose(gl.cpu().double().numpy(), logits.numpy(), rtol=1e-5, atol=2e-5)
+    assert torch.equal(gi.cpu().long(), idx), "selected experts differ from the oracle"
+    np.testing.assert_allclose(gw.cpu().double().numpy(), w.numpy(), rtol=5e-5, atol=1e-6)
+    # the (D, E) form of the same call: the same experts; logits up to the order of the sums
+    pi, pw, pl = _abi.router_topk(x, router, bias, k, score, spec.mode.renormalize, want_logits=True)
+    assert torch.equal(pi, gi)
+    np.testing.assert_allclose(gl.cpu().numpy(), pl.cpu().numpy(), rtol=1e-5, atol=2e-5)
+    # with the normalisation in front
+    g = torch.Generator().manual_seed(d)
+    gamma = (1.0 + 0.3 * torch.randn(d, generator=g)).bfloat16().to(gpu_device)
+    xn, ni, nw, nl = _abi.router_topk_norm(x, gamma, 1e-5, router, bias, k, score, spec.mode.renormalize,
+                                           want_logits=True, router_t=router_t)
+    xn2 = _abi.router_topk_norm(x, gamma, 1e-5, router, bias, k, score, spec.mode.renormalize)[0]
+    assert torch.equal(xn, xn2), "the normalised rows do not depend on the router's layout"
+    qi, qw, ql = _abi.router_topk(xn, router, bias, k, score, spec.mode.renormalize, want_logits=True,
+                                  router_t=router_t)
+    assert torch.equal(ni, qi) and torch.equal(nw, qw) and torch.equal(nl, ql)
+    # exact ties and special values: small integers make every sum exact
+    gi2 = torch.Generator().manual_seed(7)
+    xi = torch.randint(-2, 3, (tokens, d), generator=gi2).float()
+    ri = torch.randint(-1, 2, (d, e), generator=gi2).float()
+    xi[0] = 0.0
+    if e > 7:
+        ri[:, 7] = ri[:, 3]
+    want = xi.double() @ ri.double()
+    ti, _, tl = _abi.router_topk(xi.bfloat16().to(gpu_device), ri.bfloat16().to(gpu_device), None, k,
+                                 want_logits=True, router_t=ri.t().contiguous().bfloat16().to(gpu_device))
+    assert torch.equal(tl.cpu().double(), want)
+    assert torch.equal(ti.cpu().long(), O.topk_lowest_index(want, k))
+
+
+def test_router_refuses_an_expert_major_matrix_where_it_does_not_read_one(gpu_device):
+    x = torch.zeros(16, 64, dtype=torch.bfloat16, device=gpu_device)
+    r = torch.zeros(8, 64, dtype=torch.bfloat16, device=gpu_device)
+    idx = torch.empty(16, 2, dtype=torch.int32, device=gpu_device)
+    w = torch.empty(16, 2, dtype=torch.float32, device=gpu_device)
+    lib = _abi.load()
+    rc = lib.fs2moe_router_topk(x.data_ptr(), r.data_ptr(), None, 16, 64, 8, 2, _abi.dtype_code(x.dtype),
+                                _abi.SCORE_SIGMOID | _abi.ROUTER_OUT_IN, 0, idx.data_ptr(), w.data_ptr(),
+                                None, None, 0, None)
+    assert rc != 0 and b"fs2moe_router_takes_out_in" in lib.fs2moe_last_error()
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
 def test_router_ties_resolve_to_lower_expert_id(gpu_device, dtype):
     # Small-integer operands: every partial sum is exact in f32 whatever the order, so exact ties
