@@ -129,7 +129,8 @@ def time_stages(module, x, reps: int):
     for rep in range(reps + 2):
         spans = {}
         (idx, w, _), spans["router"] = timed(lambda: _abi.router_topk(
-            x, module.router, module.router_bias, module.top_k, _SCORE_FNS[module.score_fn], module.renormalize
+            x, module.router, module.router_bias, module.top_k, _SCORE_FNS[module.score_fn], module.renormalize,
+            router_t=module._router_expert_major(),  # as the module's own calls pass it
         ))
         # the row copy that the fused path skips, timed on its own (at the place in the sequence
         # where it would be the real thing): the HBM-bound part of dispatch, with its own roofline
@@ -212,15 +213,28 @@ def cpu_baseline(wl, seconds: float) -> dict:
     }
 
 
-def vendor_gemm(spec, dev) -> dict:
+def vendor_gemm(spec, dev, fp8: bool = False) -> dict:
     """The routed rows as ONE group through the vendor's dense bf16 GEMM: (T K, D) x (D, F) twice and
     (T K, F) x (F, D).  No grouping, no skew, no gather, no gate: what the same flops cost in the
     library AMD ships, on this box.  Timed twice: on data drawn like the workload's, and on all-zero
     operands, which toggle no bits in the matrix pipes and so show what the same instruction stream
-    reaches when the clock is not held down by power."""
+    reaches when the clock is not held down by power.
+    ``fp8``: both operands e4m3 with one scale per tensor (torch._scaled_mm, bf16 result): the
+    library's counterpart of the W8A8 workload's products, without that path's block scales, channel
+    scales or the quantisation of the gated product."""
     import torch
 
     rows, d, f = spec.num_tokens * spec.top_k, spec.model_dim, spec.inner_dim
+    if fp8:
+        one = torch.ones((), device=dev)
+        mm = lambda a, b: torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)  # noqa: E731
+        cast = lambda t: t.to(torch.float8_e4m3fn)  # noqa: E731
+    else:
+        mm = lambda a, b: torch.matmul(a, b)  # noqa: E731
+        cast = lambda t: t.to(torch.bfloat16)  # noqa: E731
+    # weights as (in, out) for the bf16 product (the reference's layout); the e4m3 product wants its
+    # second operand column-major, i.e. stored (out, in)
+    wshape = (lambda i, o: (o, i)) if fp8 else (lambda i, o: (i, o))
 
     def timed(fn, reps=20):
         for _ in range(10):
@@ -238,20 +252,21 @@ def vendor_gemm(spec, dev) -> dict:
         return best
 
     flops = 6.0 * rows * d * f
-    out = {"what": "torch.matmul (hipBLASLt) on the routed rows as one dense group: gate, up and down products"}
+    out = {"what": ("torch._scaled_mm (hipBLASLt, e4m3 x e4m3, per-tensor scales)" if fp8 else "torch.matmul (hipBLASLt)")
+                   + " on the routed rows as one dense group: gate, up and down products"}
     for name in ("normal", "zeros"):
         if name == "normal":
             g = torch.Generator(device=dev).manual_seed(1)
-            x = torch.randn(rows, d, device=dev, generator=g).to(torch.bfloat16)
-            h = torch.randn(rows, f, device=dev, generator=g).to(torch.bfloat16)
-            w1 = (0.02 * torch.randn(d, f, device=dev, generator=g)).to(torch.bfloat16)
-            w2 = (0.02 * torch.randn(f, d, device=dev, generator=g)).to(torch.bfloat16)
+            x = cast(torch.randn(rows, d, device=dev, generator=g))
+            h = cast(torch.randn(rows, f, device=dev, generator=g))
+            w1 = cast((1.0 if fp8 else 0.02) * torch.randn(*wshape(d, f), device=dev, generator=g))
+            w2 = cast((1.0 if fp8 else 0.02) * torch.randn(*wshape(f, d), device=dev, generator=g))
         else:
-            x, h = torch.zeros(rows, d, device=dev, dtype=torch.bfloat16), torch.zeros(rows, f, device=dev, dtype=torch.bfloat16)
-            w1, w2 = torch.zeros(d, f, device=dev, dtype=torch.bfloat16), torch.zeros(f, d, device=dev, dtype=torch.bfloat16)
+            x, h = cast(torch.zeros(rows, d, device=dev)), cast(torch.zeros(rows, f, device=dev))
+            w1, w2 = cast(torch.zeros(*wshape(d, f), device=dev)), cast(torch.zeros(*wshape(f, d), device=dev))
         with torch.no_grad():
-            up_ms = timed(lambda: torch.matmul(x, w1))
-            down_ms = timed(lambda: torch.matmul(h, w2))
+            up_ms = timed(lambda: mm(x, w1))
+            down_ms = timed(lambda: mm(h, w2))
         total = 2 * up_ms + down_ms
         ent = {"ms": round(total, 4), "gate_or_up_ms": round(up_ms, 4), "down_ms": round(down_ms, 4),
                "achieved_tflops": round(flops / (total * 1e-3) / 1e12, 1)}
@@ -516,7 +531,7 @@ def main() -> int:
     if args.training_step and spec.weight_dtype != "fp8":
         result["training_step"] = training_step(module, x3, max(3, args.steps // 10))
     if not args.no_vendor_gemm and spec.dtype == "bf16" and not experts_hbm_bound:
-        result["vendor_gemm"] = vendor_gemm(spec, dev)
+        result["vendor_gemm"] = vendor_gemm(spec, dev, fp8=w8a8)
         if spec.weight_dtype == "bf16":
             with torch.no_grad():
                 z = experts_on_zero_operands(module, x2, args.stage_reps)
