@@ -539,6 +539,13 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     constexpr int CH = ROWB / 16;           // 16-byte chunks per row
     constexpr int RPI = 64 / CH;            // rows per store instruction
     uint8_t* buf = smem_raw + (gu & 1) * UNIT_BYTES + wave * 8192;
+    // Everything below is cheap to derive from the lane number but loop-invariant: computed ahead of
+    // the main loop it would sit in registers that loop needs, or in scratch (three dwords reloaded
+    // at the start of every tile's epilogue, as the compiler had it).  An opaque copy of the lane
+    // number keeps the arithmetic here.
+    int lane_l = lane;
+    asm volatile("" : "+v"(lane_l));
+    const int lane = lane_l, lr = lane & 31, lk = lane >> 5;
     // write side: row lr, chunk 4 fn + q, half lk
     const int wkey = DUAL ? ((lr >> 1) & 7) : (lr & 15);
     const uint32_t wbase = (uint32_t)(lr * ROWB + (wkey << 4) + lk * 8);
@@ -552,11 +559,7 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     const int r_lane = lane / CH;
     const uint32_t lane_off = (uint32_t)((r_lane * ldc + n) * 2);
     const bool col_ok = n < N;
-    // The addresses below are cheap (one XOR or add each) but loop-invariant; computed ahead of the
-    // main loop they would sit in registers the MFMA loop needs, or in scratch.  An opaque copy of
-    // each base keeps them here.
-    uint32_t wbase_l = wbase, rbase_l = rbase, lane_off_l = lane_off;
-    asm volatile("" : "+v"(wbase_l), "+v"(rbase_l), "+v"(lane_off_l));
+    const uint32_t wbase_l = wbase, rbase_l = rbase, lane_off_l = lane_off;
 #pragma unroll
     for (int fm = 0; fm < 2; ++fm) {
 #pragma unroll
@@ -610,6 +613,9 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
   auto store_products = [&](const Tile& t, int gu) {
     constexpr int ROWB = 128, CH = 8, RPI = 8;
     uint8_t* buf = smem_raw + (gu & 1) * UNIT_BYTES + wave * 8192;
+    int lane_l = lane;  // (as in store_tile)
+    asm volatile("" : "+v"(lane_l));
+    const int lane = lane_l, lr = lane & 31, lk = lane >> 5;
     const uint32_t wbase = (uint32_t)(lr * ROWB + (((lr >> 1) & 7) << 4) + lk * 8);
     const uint32_t rbase = (uint32_t)((lane / CH) * ROWB + (((lane % CH) ^ (lane >> 4)) << 4));
     const int n = t.n0 + wn * 64 + (lane % CH) * 8;

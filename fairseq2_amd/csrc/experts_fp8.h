@@ -140,12 +140,17 @@ __global__ __launch_bounds__(256, DUAL ? 4 : 3) void glu_gemm_fp8w_kernel(
 
   const int cg = wave / KS, ks = wave % KS;  // set of channel groups in the block, part of K
   const int groups = N / 16;                 // N is a multiple of 16
-  const int ln = lane & 15, g = lane >> 4;
   const int nkb = Kdim / 64;  // the host guarantees Kdim % 64 == 0
   const size_t group_stride = (size_t)Kdim * 16;  // bytes between the tiles of consecutive groups
   const int kb_lo = ks * nkb / KS, kb_hi = (ks + 1) * nkb / KS;
 
   for (int item = blockIdx.x; item < total; item += gridDim.x) {
+    // (what follows from the lane number is worked out per item from an opaque copy of it: hoisted
+    // out of this loop, the addresses' lane parts took registers the inner loop has no room for and
+    // were spilled to scratch and reloaded for every item)
+    int lane_l = tid & 63;
+    asm volatile("" : "+v"(lane_l));
+    const int lane = lane_l, ln = lane & 15, g = lane >> 4;
     // expert of the item (wave-uniform)
     int e = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
