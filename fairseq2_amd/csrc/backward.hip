@@ -94,7 +94,8 @@ __global__ __launch_bounds__(wgk::WAVES * 64) void grouped_wgrad_kernel(
   const bool dense = g.counts == nullptr;
   // Grouped: the experts are taken in descending order of their row counts (ties: lower index
   // first), so that the longest chains of chunks start first and the short ones fill the end of the
-  // launch.  Every block finds the expert of its rank itself: E <= 256 counts, one comparison loop.
+  // launch.  Every block finds the expert of its rank itself: a thread per expert, one comparison loop over
+  // the E counts (the block has 768 threads, the library's limit is 512 experts).
   // One group: the rows are cut into segments of seg_rows, one slot each, whose partial sums go to
   // `partial` [segments, M, N] in f32 for wgrad_reduce_kernel to add in order.
   int e = 0, off, cnt;

@@ -63,7 +63,8 @@ constexpr int RING_BYTES = 2 * UNIT_BYTES;         // 128 KB
 #endif
 constexpr int BAND = FS2MOE_GEMM_BAND;  // row blocks per band of the tile order (see locate)
 constexpr int LIGHT_ROWS = 128;  // a last tile of at most this many rows costs about half a tile
-// after the ring: heavy-tile prefix [257], light-tile prefix [257], counts [256], offsets [256]
+// after the ring: heavy-tile prefix [E + 1], light-tile prefix [E + 1], counts [E], offsets [E], each
+// sized for the library's limit on E
 constexpr int TABLE_INTS = 4 * FS2MOE_MAX_EXPERTS + 8;
 // then, for e4m3 weights, the per-channel scales of two tiles (the one being multiplied and the one
 // whose loads are under way): [2][256] f32

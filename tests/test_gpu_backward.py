@@ -520,6 +520,8 @@ def _reference_gradients(wl, grad_out, residual, activation=None):
         ("softmax_renorm_output", True, 1.0, False, dict(tokens=1, model_dim=192, num_experts=24, top_k=4, inner_dim=128)),
         # one selected expert with renormalised weights: w = 1 whatever the logits, a zero router gradient
         ("sigmoid_renorm_output", True, 1.0, True, dict(tokens=257, model_dim=192, num_experts=8, top_k=1, inner_dim=64)),
+        # past 256 experts and top-16 (the backward kernels' tables and per-token loops at the library's limits)
+        ("softmax_renorm_output", False, 1.0, False, dict(tokens=70, model_dim=64, num_experts=384, top_k=24, inner_dim=32)),
     ],
 )
 def test_layer_gradients_match_autograd_of_the_reference(gpu_device, dtype, mode, shared, zipf, with_residual, shape):
