@@ -285,8 +285,26 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     // the two LDS slots it goes to (tiles alternate)
     float ld_scale = 0.f;
     int ld_tiles = 0;
-    auto setup_loads = [&](int j) {
-      const Tile t = locate(j);
+    // The tile after the one set up last, looked up a tile ahead: which tile it is, and (fused
+    // gather) the tokens its rows are read from.  Those come out of row_map, a load that the tile's
+    // own loads depend on; asked for when the tile before it is set up, they have long arrived when
+    // the tile's turn comes, and its first unit goes out without a round trip to memory in front.
+    Tile pre_t = {0, 0, 0, 0};
+    int pre_rows[8];
+    auto lookup_ahead = [&](int j) {
+      pre_t = locate(j);
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const int row = 8 * (q + 4 * jj) + (lane >> 3);
+        int grow = pre_t.row0 + row;
+        grow = grow < pre_t.row_end ? grow : pre_t.row_end - 1;  // clamped rows are never stored
+        // fused gather: logical row r of the activations is row row_map[r] of A (rows below row_end
+        // are real pairs, so their map entries are tokens, never the -1 of padding)
+        pre_rows[jj] = row_map != nullptr ? row_map[grow] : grow;
+      }
+    };
+    auto setup_loads = [&]() {
+      const Tile t = pre_t;
       if constexpr (FP8) {
         // wstride counts codes = bytes here; the pointers stay typed as 16-bit
         ld_bg = reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(B0) +
@@ -309,12 +327,7 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
         const int p = q + 4 * jj;
         const int row = 8 * p + (lane >> 3), slot = lane & 7;
         const int kc = slot ^ ((row >> 1) & 7);
-        int grow = t.row0 + row;
-        grow = grow < t.row_end ? grow : t.row_end - 1;  // clamped rows are never stored
-        // fused gather: logical row r of the activations is row row_map[r] of A (rows below row_end
-        // are real pairs, so their map entries are tokens, never the -1 of padding)
-        if (row_map != nullptr) grow = row_map[grow];
-        pa[jj] = (uint32_t)(((size_t)grow * lda + kc * 8) * 2);
+        pa[jj] = (uint32_t)(((size_t)pre_rows[jj] * lda + kc * 8) * 2);
       }
       // piece p holds rows 8p .. 8p+7; pieces past the tile's last row are not loaded (the consumer
       // waves that would read them are idle)
@@ -436,9 +449,15 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     };
     TileOrder order(my_heavy, my_tiles - my_heavy, (int)(blockIdx.x & 7));
     int ld_ku = -1;  // unit (within its tile) loaded last
+    int looked_up = 1;  // tiles looked up so far
+    lookup_ahead(order.next());
     auto load_next = [&]() {
       if (ld_ku < 0 || ld_ku + 1 == nu) {
-        setup_loads(order.next());
+        setup_loads();
+        if (looked_up < my_tiles) {
+          lookup_ahead(order.next());
+          ++looked_up;
+        }
         ld_ku = 0;
       } else {
         ++ld_ku;
