@@ -49,6 +49,35 @@ def test_abi_version_and_limits(lib):
         assert re.search(rf"#define {name} {val}\b", text)
 
 
+def test_expert_major_router_is_taken_where_the_library_says_so(lib):
+    """ROUTER_OUT_IN: the size rule of fs2moe_router_takes_out_in, the wrapper's choice between the two
+    forms, its shape check, and the refusal of the flag elsewhere (host code only)."""
+    assert re.search(rf"#define FS2MOE_ROUTER_OUT_IN {hex(_abi.ROUTER_OUT_IN)}\b", open(HEADER).read())
+    takes = lib.fs2moe_router_takes_out_in
+    assert takes(8192, 2048, 128, _abi.BF16) == 1 and takes(8192, 2048, 128, _abi.F32) == 0
+    assert takes(8192, 2048 + 64, 128, _abi.BF16) == 0, "whole steps of 128 features"
+    assert takes(8192, 2048, 132, _abi.BF16) == 0 and takes(8192, 2048, 264, _abi.BF16) == 0
+    assert takes(32, 2048, 128, _abi.BF16) == 0 and takes(64, 2048, 128, _abi.BF16) == 0
+    assert takes(4097, 2048, 128, _abi.BF16) == 1 and takes(33, 128, 8, _abi.BF16) == 1
+    x = torch.zeros(8192, 256, dtype=torch.bfloat16)
+    r = torch.zeros(256, 16, dtype=torch.bfloat16)
+    rt = r.t().contiguous()
+    assert _abi.router_operand(lib, x, r, None, _abi.SCORE_SOFTMAX) == (r, _abi.SCORE_SOFTMAX)
+    mat, score = _abi.router_operand(lib, x, r, rt, _abi.SCORE_SOFTMAX)
+    assert mat is rt and score == (_abi.SCORE_SOFTMAX | _abi.ROUTER_OUT_IN)
+    mat, score = _abi.router_operand(lib, x[:16], r, rt, _abi.SCORE_SIGMOID)
+    assert mat is r and score == _abi.SCORE_SIGMOID, "few tokens: the (D, E) form"
+    with pytest.raises(ValueError, match="router_t"):
+        _abi.router_operand(lib, x, r, r, _abi.SCORE_SOFTMAX)  # not transposed
+    with pytest.raises(ValueError, match="router_t"):
+        _abi.router_operand(lib, x, r, rt.float(), _abi.SCORE_SOFTMAX)
+    fake = ctypes.c_void_p(0x1000)
+    rc = lib.fs2moe_router_topk(fake, fake, None, 16, 256, 16, 2, _abi.BF16, _abi.SCORE_SIGMOID | _abi.ROUTER_OUT_IN,
+                                0, fake, fake, None, None, 0, None)
+    assert rc == -1 and b"fs2moe_router_takes_out_in" in lib.fs2moe_last_error()
+    assert _abi.router_expert_major(torch.zeros(4, 4)) is None, "no copy of what is not a bf16 matrix on the GPU"
+
+
 def test_argument_errors_are_reported_without_touching_the_gpu(lib):
     # null pointers
     rc = lib.fs2moe_router_topk(None, None, None, 4, 8, 4, 2, _abi.BF16, 0, 0, None, None, None, None, 0, None)
