@@ -294,7 +294,13 @@ def router_expert_major(router: Tensor, holder=None) -> Tensor | None:
     if router.dtype != torch.bfloat16 or not router.is_cuda:
         return None
     holder = router if holder is None else holder
-    key = (router._version, router.data_ptr(), tuple(router.shape))
+    try:
+        version = router._version
+    except RuntimeError:
+        # a tensor made under torch.inference_mode() has no version counter: nothing would say when
+        # it has been written to, so no copy is kept and the router reads the matrix as it is
+        return None
+    key = (version, router.data_ptr(), tuple(router.shape))
     hit = getattr(holder, "_fs2moe_router_t", None)
     if hit is None or hit[0] != key:
         with torch.no_grad():

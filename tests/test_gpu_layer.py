@@ -414,6 +414,10 @@ def test_expert_major_copy_of_the_router_follows_the_parameter(gpu_device):
         assert float(_abi.router_expert_major(r)[0, 0]) == float(i)
         del r
     assert _abi.router_expert_major(torch.zeros(4, 4, device=gpu_device)) is None, "f32: no copy"
+    with torch.inference_mode():
+        made_here = torch.zeros(128, 8, dtype=torch.bfloat16, device=gpu_device)
+        assert _abi.router_expert_major(made_here) is None, "no version counter to watch: no copy"
+        assert torch.equal(m(x), after), "a module made outside runs inside inference mode as before"
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
