@@ -202,118 +202,125 @@ __global__ __launch_bounds__(mx::NWAVES * 64) void glu_gemm_mx_kernel(
 
   if (wave >= CONSUMERS) {
     // ---- producers ----------------------------------------------------------------------------------
-    // Producer q moves pieces q, q + 4, ... of both operands: an activation piece is 8 rows x 128 B
-    // (lane i: row i / 8, 16-byte slot i % 8, fetching the chunk that the swizzle puts there), a
-    // weight piece is one 1 KB tile of 16 channels x 64 k, which lands in its channels' 128-byte
-    // rows as chunks 4 kb .. 4 kb + 3 (kb = the tile's half of the unit).  Plus the unit's four scale
-    // bytes of rows 64 q .. 64 q + 63 (one dword per lane) and, with a tile's first unit, its
-    // channel scales.
+    // Producer q moves pieces q, q + 4, ... of both operands, 8 rows x 128 B each, straight from
+    // global memory into LDS (buffer_load ... lds: lane i's 16 bytes land at 16 i of the piece, i.e.
+    // row i / 8, slot i % 8, and the lane fetches the chunk that the swizzle puts there): no staging
+    // registers and no LDS store instructions.  An activation piece is 8 rows of the (gathered)
+    // operand; a weight piece is 8 channel rows of a 16-channel group, each row made of 64 bytes of
+    // the group's two 1 KB tiles (16 channels x 64 k) of this unit.  Plus the unit's four scale bytes
+    // of rows 64 q .. 64 q + 63 (a dword per lane, the same way) and, with a tile's first unit, its
+    // channel scales.  The loads of unit u + 1 go out when the consumers are done with unit u - 1 (the
+    // barrier of unit u) and must have landed by the next barrier: one unit of lead, so nothing may
+    // stand between that barrier and the loads.  A tile's addresses are therefore worked out a tile
+    // ahead (which tile, the tokens of its rows, its channel scale: lookup_ahead).
+    // Against producers that stage through registers and store to LDS (same box, rocprofv3, Qwen3
+    // prefill layer): gate/up 247.3 -> 241.5 us, down 164.0 -> 163.2 us; harness, random codes:
+    // Mixtral's counts 2723 -> 2635 us, Scout's 1242 -> 1220, Qwen3's 470 -> 458.  (Without the
+    // look-ahead the same producers were slower in the layer: 241 -> 247 and 158 -> 170 us.)
     const int q = wave - CONSUMERS;
+    typedef __attribute__((address_space(3))) void* lds_ptr;
     uint32_t pa[8], pb[8], ps = 0;
     int a_pieces = 0;
     const uint8_t* ld_b[2] = {B0, B0};
     float ld_scale = 0.f;
     int ld_tiles = 0;
-    auto setup_loads = [&](int j) {
-      const Tile t = locate(j);
-      ld_b[0] = B0 + (size_t)t.e * wstride;
-      ld_b[1] = DUAL ? B1 + (size_t)t.e * wstride : ld_b[0];
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(A), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t as_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(As), 0, -1, 0x00020000);
+    // The tile after the one set up last, looked up a tile ahead: which tile it is, the tokens its
+    // rows are read from (row_map: loads that the tile's own loads depend on) and its channel scale.
+    Tile pre_t = {0, 0, 0, 0};
+    int pre_rows[8], pre_srow = 0;
+    float pre_scale = 0.f;
+    auto lookup_ahead = [&](int j) {
+      pre_t = locate(j);
       {
         const int v = 64 * q + lane;  // virtual channel: gate 0..127, up 128..255
         const bool up = DUAL && v >= 128;
-        int ch = t.n0 + (up ? v - 128 : v);
+        int ch = pre_t.n0 + (up ? v - 128 : v);
         ch = ch < N ? ch : N - 1;  // clamped channels are never stored
-        ld_scale = (up ? S1 : S0)[(size_t)t.e * N + ch];
-        ++ld_tiles;
+        pre_scale = (up ? S1 : S0)[(size_t)pre_t.e * N + ch];
       }
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
-        const int p = q + 4 * jj;
-        const int row = 8 * p + (lane >> 3), slot16 = lane & 7;
+        int grow = pre_t.row0 + 8 * (q + 4 * jj) + (lane >> 3);
+        grow = grow < pre_t.row_end ? grow : pre_t.row_end - 1;  // clamped rows are never stored
+        pre_rows[jj] = row_map != nullptr ? row_map[grow] : grow;
+      }
+      int grow = pre_t.row0 + 64 * q + lane;
+      grow = grow < pre_t.row_end ? grow : pre_t.row_end - 1;
+      pre_srow = row_map != nullptr ? row_map[grow] : grow;
+    };
+    auto setup_loads = [&]() {
+      const Tile t = pre_t;
+      ld_b[0] = B0 + (size_t)t.e * wstride;
+      ld_b[1] = DUAL ? B1 + (size_t)t.e * wstride : ld_b[0];
+      ld_scale = pre_scale;
+      ++ld_tiles;
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const int row = 8 * (q + 4 * jj) + (lane >> 3), slot16 = lane & 7;
         const int kc = slot16 ^ ((row >> 1) & 7);
-        int grow = t.row0 + row;
-        grow = grow < t.row_end ? grow : t.row_end - 1;  // clamped rows are never stored
-        if (row_map != nullptr) grow = row_map[grow];
-        pa[jj] = (uint32_t)((size_t)grow * Kdim + kc * 16);
+        pa[jj] = (uint32_t)((size_t)pre_rows[jj] * Kdim + kc * 16);
       }
-      {
-        int grow = t.row0 + 64 * q + lane;
-        grow = grow < t.row_end ? grow : t.row_end - 1;
-        if (row_map != nullptr) grow = row_map[grow];
-        ps = (uint32_t)grow * 4u;
-      }
+      ps = (uint32_t)pre_srow * 4u;
       const int rows = t.row_end - t.row0;
       a_pieces = rows >= BM ? 8 : (rows - 8 * q + 31) / 32;
       a_pieces = a_pieces < 0 ? 0 : a_pieces;
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
-        // piece p: channel group gi = p / 2 of the 16 virtual groups, half kb = p % 2 of the unit
-        const int p = q + 4 * jj;
-        const int gi = p >> 1, kb = p & 1;
+        const int P = q + 4 * jj;
+        const int gi = P >> 1, r16 = 8 * (P & 1) + (lane >> 3);
+        const int row = 8 * P + (lane >> 3);
+        const int c = (lane & 7) ^ ((row >> 1) & 7);
         int group = t.n0 / 16 + (DUAL ? (gi & 7) : gi);
         group = group < N / 16 ? group : N / 16 - 1;  // clamped channels are never stored
-        pb[jj] = (uint32_t)(((size_t)group * nkb + kb) * 1024 + mx_tile_row(lane) * 64 + (lane & 3) * 16);
+        pb[jj] = (uint32_t)(((size_t)group * nkb + (c >> 2)) * 1024 + r16 * 64 + (c & 3) * 16);
       }
     };
-    u32x4 stage[16];
-    uint32_t stage_s = 0;
-    int stage_pieces = 0;
-    int stage_scale_slot = -1;
-    float stage_scale = 0.f;
-    auto load_unit = [&](int ku) {
-      const uint8_t* abase = A + (size_t)ku * UK;
+    auto issue_unit = [&](int ku, int half) {
+      uint8_t* base = smem_raw + half * UNIT_BYTES;
+      const uint32_t koff_a = (uint32_t)ku * UK;
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj)
-        if (jj < a_pieces) stage[jj] = *reinterpret_cast<const u32x4*>(abase + pa[jj]);
-      stage_s = *reinterpret_cast<const uint32_t*>(As + (size_t)ku * a_rows * 4 + ps);
-      const size_t koff = (size_t)ku * 2048;  // two tiles along k per unit
+        if (jj < a_pieces)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(base + (q + 4 * jj) * 1024), 16, pa[jj], koff_a, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(as_rsrc, (lds_ptr)(&s_ascale[half * BM + 64 * q]), 4, ps,
+                                               (uint32_t)ku * (uint32_t)a_rows * 4u, 0, 0);
+      const __amdgpu_buffer_rsrc_t bg = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_b[0]), 0, -1, 0x00020000);
+      const __amdgpu_buffer_rsrc_t bu = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_b[1]), 0, -1, 0x00020000);
+      const uint32_t koff_w = (uint32_t)ku * 2048u;  // two tiles along k per unit
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
-        // pieces q + 4 jj: groups 0..7 (jj < 4) are gate channels when DUAL, the rest up channels
-        const uint8_t* b = (DUAL && jj >= 4) ? ld_b[1] : ld_b[0];
-        stage[8 + jj] = *reinterpret_cast<const u32x4*>(b + koff + pb[jj]);
+        if (DUAL && jj >= 4)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(bu, (lds_ptr)(base + A_BYTES + (q + 4 * jj) * 1024), 16, pb[jj], koff_w, 0, 0);
+        else
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(bg, (lds_ptr)(base + A_BYTES + (q + 4 * jj) * 1024), 16, pb[jj], koff_w, 0, 0);
       }
-      stage_pieces = a_pieces;
-      stage_scale_slot = ku == 0 ? ((ld_tiles - 1) & 1) : -1;
-      stage_scale = ld_scale;
-    };
-    auto write_unit = [&](int half) {
-      uint8_t* dst = smem_raw + half * UNIT_BYTES + q * 1024 + lane * 16;
-#pragma unroll
-      for (int jj = 0; jj < 8; ++jj)
-        if (jj < stage_pieces) *reinterpret_cast<u32x4*>(dst + jj * 4096) = stage[jj];
-      s_ascale[half * BM + 64 * q + lane] = stage_s;
-      // tile piece p = q + 4 jj: channel rows 16 (p / 2) + mx_tile_row(lane), chunk 4 (p % 2) +
-      // lane % 4 of the row, in slot chunk ^ ((row >> 1) & 7); 16 (p / 2) does not change the key
-      const int r = mx_tile_row(lane), key = (r >> 1) & 7;
-      const int kc = 4 * (q & 1) + (lane & 3);  // p % 2 == q % 2
-      uint8_t* wdst = smem_raw + half * UNIT_BYTES + A_BYTES + ((kc ^ key) << 4);
-#pragma unroll
-      for (int jj = 0; jj < 8; ++jj) {
-        const int gi = (q + 4 * jj) >> 1;
-        *reinterpret_cast<u32x4*>(wdst + (16 * gi + r) * 128) = stage[8 + jj];
-      }
-      if (stage_scale_slot >= 0) s_wscale[stage_scale_slot * BNV + 64 * q + lane] = stage_scale;
+      if (ku == 0) s_wscale[((ld_tiles - 1) & 1) * BNV + 64 * q + lane] = ld_scale;
     };
     TileOrder order(my_heavy, my_tiles - my_heavy, (int)(blockIdx.x & 7));
-    int ld_ku = -1;
-    auto load_next = [&]() {
-      if (ld_ku < 0 || ld_ku + 1 == nu) {
-        setup_loads(order.next());
+    int ld_ku = -1, looked_up = 1;
+    lookup_ahead(order.next());
+    auto issue_next = [&](int half) {
+      const bool first = ld_ku < 0 || ld_ku + 1 == nu;
+      if (first) {
+        setup_loads();
         ld_ku = 0;
       } else {
         ++ld_ku;
       }
-      load_unit(ld_ku);
+      issue_unit(ld_ku, half);
+      if (first && looked_up < my_tiles) {  // (after the unit's loads have gone out)
+        lookup_ahead(order.next());
+        ++looked_up;
+      }
     };
-    load_next();
-    write_unit(0);
-    if (1 < total_units) load_next();
+    issue_next(0);
     int ku = 0;
     for (int gu = 0; gu < total_units; ++gu) {
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of unit gu has landed
       __syncthreads();  // unit gu is in LDS; the consumers are done with unit gu - 1
-      if (gu + 1 < total_units) write_unit((gu + 1) & 1);
-      if (gu + 2 < total_units) load_next();
+      if (gu + 1 < total_units) issue_next((gu + 1) & 1);
       if (++ku == nu) {
         ku = 0;
         __syncthreads();  // the consumers' barrier ahead of their epilogue
