@@ -12,7 +12,8 @@
 // Persistence.  One block per CU walks a list of output tiles, dealt out so that every block gets
 // the same amount of work and the blocks of an XCD work on neighbouring tiles (see the tile tables
 // below).  The tile -> (expert, rows) map comes from counts/offsets, copied to LDS once; nothing is
-// read back to the host.
+// read back to the host.  Tiles that would make up a last round of a few whole tiles are dealt as
+// halves (128 rows) when that lets the round end in a light tile's time.
 //
 // Pipeline.  K is walked in units of 64: a unit is a 256 x 64 activation block (128-byte rows: a
 // 64-byte piece of a row would make the L1 fetch every 128-byte line twice and halve the fill rate)
@@ -205,13 +206,24 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
   }
   // The host guarantees that the number of tiles fits 31 bits.
   const int total_heavy = s_hstart[E];
-  const int real = (total_heavy + s_lstart[E]) * n_tiles;
   const int slot = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   const int grid = (int)gridDim.x;
+  // The heavy tiles that do not fill a round of the deal (one tile per block) would hold their
+  // blocks for a whole tile's time while the others idle.  When both halves of each of them and all
+  // light tiles fit ONE round, they are dealt as halves of 128 rows (rows 0..127 and 128..255 of the
+  // tile, each a light tile's work): the last round then takes a light tile's time.  Every output
+  // element is still the same sum in the same order.
+  const int all_heavy = total_heavy * n_tiles;
+  const int lights = s_lstart[E] * n_tiles;
+  const int rest = all_heavy % grid;
+  const int split = 2 * rest + lights <= grid ? rest : 0;
+  // list order: heavy tiles [0, heavy_end), halves [heavy_end, halves_end), light tiles after that
+  const int heavy_end = all_heavy - split;
+  const int halves_end = heavy_end + 2 * split;
+  const int real = halves_end + lights;
   const int my_tiles = slot < real ? (real - slot + grid - 1) / grid : 0;
   if (my_tiles == 0) return;
   // of which heavy: the block's j-th tile (in list order) is heavy for j < my_heavy
-  const int heavy_end = total_heavy * n_tiles;
   const int my_heavy = slot < heavy_end ? (heavy_end - slot + grid - 1) / grid : 0;
 
   // units per tile; the host guarantees Kdim % 64 == 0
@@ -223,9 +235,13 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
     int e, row0, row_end, n0;
   };
   auto locate = [&](int j) {
-    const int logical = slot + j * grid;
-    const bool is_light = logical >= heavy_end;
-    const int in_kind = is_light ? logical - heavy_end : logical;
+    const int listed = slot + j * grid;
+    const bool is_light = listed >= halves_end;
+    // a half names its heavy tile: the halves of heavy tile heavy_end + i are listed at
+    // heavy_end + 2 i and + 2 i + 1
+    const int half = (listed >= heavy_end && !is_light) ? ((listed - heavy_end) & 1) : -1;
+    const int logical = half >= 0 ? heavy_end + ((listed - heavy_end) >> 1) : listed;
+    const int in_kind = is_light ? listed - halves_end : logical;
     int mt = in_kind / n_tiles;  // m-tile in list order: which expert
     const int32_t* start = is_light ? s_lstart : s_hstart;
     int found = 0;
@@ -257,10 +273,15 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
       nt = t / gm;
       first_row = (b * BAND + t - nt * gm) * BM;
     }
+    int last_row = cnt;
+    if (half >= 0) {
+      first_row += half * LIGHT_ROWS;
+      last_row = last_row < first_row + LIGHT_ROWS ? last_row : first_row + LIGHT_ROWS;
+    }
     Tile t;
     t.e = found;
     t.row0 = __builtin_amdgcn_readfirstlane(off + first_row);
-    t.row_end = __builtin_amdgcn_readfirstlane(off + cnt);
+    t.row_end = __builtin_amdgcn_readfirstlane(off + last_row);
     t.n0 = __builtin_amdgcn_readfirstlane(nt) * BN;
     return t;
   };

@@ -146,12 +146,20 @@ __global__ __launch_bounds__(mx::NWAVES * 64) void glu_gemm_mx_kernel(
     __syncthreads();
   }
   const int total_heavy = s_hstart[E];
-  const int real = (total_heavy + s_lstart[E]) * n_tiles;
   const int slot = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   const int grid = (int)gridDim.x;
+  // the heavy tiles left over by the whole rounds of the deal go out as halves of 128 rows when
+  // those and the light tiles fit one round (as in the bf16 kernel: same sums, a shorter last round)
+  const int all_heavy = total_heavy * n_tiles;
+  const int lights = s_lstart[E] * n_tiles;
+  const int rest = all_heavy % grid;
+  const int split = 2 * rest + lights <= grid ? rest : 0;
+  // list order: heavy tiles [0, heavy_end), halves [heavy_end, halves_end), light tiles after that
+  const int heavy_end = all_heavy - split;
+  const int halves_end = heavy_end + 2 * split;
+  const int real = halves_end + lights;
   const int my_tiles = slot < real ? (real - slot + grid - 1) / grid : 0;
   if (my_tiles == 0) return;
-  const int heavy_end = total_heavy * n_tiles;
   const int my_heavy = slot < heavy_end ? (heavy_end - slot + grid - 1) / grid : 0;
   const int nu = Kdim / UK;  // the host guarantees Kdim % 128 == 0
   const int total_units = my_tiles * nu;
@@ -160,9 +168,11 @@ __global__ __launch_bounds__(mx::NWAVES * 64) void glu_gemm_mx_kernel(
     int e, row0, row_end, n0;
   };
   auto locate = [&](int j) {
-    const int logical = slot + j * grid;
-    const bool is_light = logical >= heavy_end;
-    const int in_kind = is_light ? logical - heavy_end : logical;
+    const int listed = slot + j * grid;
+    const bool is_light = listed >= halves_end;
+    const int half = (listed >= heavy_end && !is_light) ? ((listed - heavy_end) & 1) : -1;
+    const int logical = half >= 0 ? heavy_end + ((listed - heavy_end) >> 1) : listed;
+    const int in_kind = is_light ? listed - halves_end : logical;
     int mt = in_kind / n_tiles;
     const int32_t* start = is_light ? s_lstart : s_hstart;
     int found = 0;
@@ -189,10 +199,15 @@ __global__ __launch_bounds__(mx::NWAVES * 64) void glu_gemm_mx_kernel(
       nt = t / gm;
       first_row = (b * BAND + t - nt * gm) * BM;
     }
+    int last_row = cnt;
+    if (half >= 0) {
+      first_row += half * LIGHT_ROWS;
+      last_row = last_row < first_row + LIGHT_ROWS ? last_row : first_row + LIGHT_ROWS;
+    }
     Tile t;
     t.e = found;
     t.row0 = __builtin_amdgcn_readfirstlane(off + first_row);
-    t.row_end = __builtin_amdgcn_readfirstlane(off + cnt);
+    t.row_end = __builtin_amdgcn_readfirstlane(off + last_row);
     t.n0 = __builtin_amdgcn_readfirstlane(nt) * BN;
     return t;
   };
