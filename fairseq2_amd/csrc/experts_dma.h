@@ -485,14 +485,76 @@ __global__ __launch_bounds__(dma::NWAVES * 64) void glu_gemm_bf16_dma_kernel(
       }
       load_unit(ld_ku);
     };
+    // bf16 weights: write_unit and load_next in one pass, register by register -- the store of a
+    // register into the ring, then the load of the next unit's piece into that register.  A wave
+    // issues in order, and its LDS stores and its loads each take their turn at a unit of the CU that
+    // it shares with the other producers (16 stores of 1 KB: about 1250 clocks next to the
+    // consumers' reads; 16 loads: about 630): as two phases one after the other they add up,
+    // interleaved the two units work at the same time.
+    auto write_and_load = [&](int half) {
+      if (ld_ku < 0 || ld_ku + 1 == nu) {
+        setup_loads();
+        if (looked_up < my_tiles) {
+          lookup_ahead(order.next());
+          ++looked_up;
+        }
+        ld_ku = 0;
+      } else {
+        ++ld_ku;
+      }
+      if constexpr (!FP8) {
+        int ku = ld_ku;
+        const bool second = TWO_SRC && ku >= nu / 2;
+        if constexpr (TWO_SRC) ku = second ? ku - nu / 2 : ku;
+        const uint16_t* a_src = second ? reinterpret_cast<const uint16_t*>(S0) : A;
+        const uint8_t* abase = reinterpret_cast<const uint8_t*>(a_src + (size_t)ku * (2 * BK));
+        uint8_t* dst = smem_raw + half * UNIT_BYTES + q * 1024 + lane * 16;
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+          if (jj < stage_pieces) *reinterpret_cast<u32x4*>(dst + jj * 4096) = stage[jj];
+          if (jj < a_pieces) stage[jj] = *reinterpret_cast<const u32x4*>(abase + pa[jj]);
+        }
+        if constexpr (KN) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const size_t k0 = ((size_t)ku * 2 + h) * BK * N;
+            const uint8_t* bg = reinterpret_cast<const uint8_t*>(ld_bg + k0);
+            const uint8_t* bu = reinterpret_cast<const uint8_t*>(ld_bu + k0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              *reinterpret_cast<u32x4*>(dst + A_BYTES + (4 * h + i) * 4096) = stage[8 + 4 * h + i];
+              stage[8 + 4 * h + i] = *reinterpret_cast<const u32x4*>((i < 2 ? bg : bu) + pb[i]);
+            }
+          }
+        } else {
+          const uint8_t* bg =
+              reinterpret_cast<const uint8_t*>((second ? ld_bu : ld_bg) + (size_t)ku * (2 * BK));
+          const uint8_t* bu =
+              TWO_SRC ? bg : reinterpret_cast<const uint8_t*>(ld_bu + (size_t)ku * (2 * BK));
+#pragma unroll
+          for (int jj = 0; jj < 8; ++jj) {
+            *reinterpret_cast<u32x4*>(dst + A_BYTES + jj * 4096) = stage[8 + jj];
+            stage[8 + jj] = *reinterpret_cast<const u32x4*>((jj < 4 ? bg : bu) + pb[jj]);
+          }
+        }
+        stage_pieces = a_pieces;
+      }
+    };
     load_next();
     write_unit(0);
     if (1 < total_units) load_next();
     int ku = 0;
     for (int gu = 0; gu < total_units; ++gu) {
       __syncthreads();  // unit gu is in LDS; the consumers are done with unit gu - 1
-      if (gu + 1 < total_units) write_unit((gu + 1) & 1);
-      if (gu + 2 < total_units) load_next();
+      if constexpr (FP8) {
+        if (gu + 1 < total_units) write_unit((gu + 1) & 1);
+        if (gu + 2 < total_units) load_next();
+      } else {
+        if (gu + 2 < total_units)
+          write_and_load((gu + 1) & 1);
+        else if (gu + 1 < total_units)
+          write_unit((gu + 1) & 1);
+      }
       if (++ku == nu) {
         ku = 0;
         __syncthreads();  // the consumers' barrier ahead of their epilogue
