@@ -30,13 +30,13 @@ MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3, "fp8": 5000.0}  # dense, publ
 # `--pmc WRITE_SIZE` runs of this script (see profiles/); None until measured for a workload.
 # The commit whose kernels the table below was measured on: a kernel change after it makes the
 # figures stale until the counter runs are repeated (the roofline object carries the stamp).
-MEASURED_TRAFFIC_AT = "2ccaa57"
+MEASURED_TRAFFIC_AT = "06e32e2"
 MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     # profiles/bench_<workload>_all_kernels.md, the two launches of the grouped experts together
     # (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0 against a 256 MiB copy)
-    "qwen3_30b_a3b": 2.628e9,     # gate/up 1542 + 101 MB, down 717 + 269 MB
-    "mixtral_8x7b": 14.800e9,     # gate/up 10152 + 470 MB, down 4044 + 134 MB
-    "llama4_scout": 6.632e9,      # routed experts only: gate/up 4220 + 134 MB, down 2193 + 84 MB
+    "qwen3_30b_a3b": 2.653e9,     # gate/up 1566 + 101 MB, down 717 + 269 MB
+    "mixtral_8x7b": 13.402e9,     # gate/up 8792 + 470 MB, down 4006 + 134 MB
+    "llama4_scout": 6.677e9,      # routed experts only: gate/up 4103 + 135 MB, down 2355 + 84 MB
     "small_fp32": 0.866e9,        # gate/up 402 + 46 MB, down 401 + 17 MB
     "qwen3_decode_fp8": 0.221e9,  # gate/up 143 + 1 MB, down 76 + 2 MB
     "qwen3_30b_a3b_fp8": 1.886e9,  # gate/up 1033 + 101 MB, down 484 + 269 MB
