@@ -15,11 +15,12 @@ from torch import Tensor
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfs2moe.so")
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
-ROUTER_OUT_IN = 0x100  # OR-ed into score_fn: the router argument is (E, D)
+ROUTER_OUT_IN = 0x100
+ACT_MXFP8 = 0x100  # OR-ed into a whole-layer call's w_dtype next to e4m3 weights: W8A8  # OR-ed into score_fn: the router argument is (E, D)
 W_IN_OUT, W_OUT_IN = 0, 1
 MAX_EXPERTS, MAX_TOP_K = 512, 32
 
@@ -977,9 +978,12 @@ def forward(
     residual: Tensor | None = None,
     norm: tuple[Tensor | None, float] | None = None,
     router_t: Tensor | None = None,
+    act_quant: bool = False,
 ) -> Tensor:
     """The whole layer through ``fs2moe_forward``: one call, intermediates in one workspace.
     ``router_t``: optionally the router matrix expert-major, (E, D), used where the library reads it.
+    ``act_quant`` (with ``scales``, i.e. e4m3 weights): the expert products on the fp8 matrix pipe,
+    the rows rounded to block-scaled e4m3 inside the call (``FS2MOE_ACT_MXFP8``).
     With ``residual`` ``(T, D)`` the result is ``residual + layer(x)`` from the same accumulation.
     With ``norm`` = (weight or None, eps) the rows are RMS-normalised on the way into the router
     (``fs2moe_forward_norm``): the result is ``[residual +] layer(rms_norm(x))``.
@@ -989,6 +993,8 @@ def forward(
     """
     lib = load()
     t, d = x.shape
+    if act_quant and scales is None:
+        raise ValueError("act_quant goes with e4m3 weights (scales)")
     if scales is None:
         f = w_down.shape[0] // num_experts
     else:
@@ -1010,7 +1016,8 @@ def forward(
     tail = (
         _ptr(residual), _ptr(mat), _ptr(router_bias), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(sg),
         _ptr(su), _ptr(sd), _ptr(hg), _ptr(hu), _ptr(hd), t, d, num_experts, top_k, f, f_shared,
-        tile_m, dtype_code(x.dtype), dtype_code(w_gate.dtype), score_fn, int(renormalize),
+        tile_m, dtype_code(x.dtype), dtype_code(w_gate.dtype) | (ACT_MXFP8 if act_quant else 0),
+        score_fn, int(renormalize),
         int(scale_input), _ptr(workspace), workspace.numel(), _ptr(out), _stream(),
     )
     if norm is None:

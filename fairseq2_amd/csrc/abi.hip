@@ -48,12 +48,15 @@ struct ForwardBuffers {
   int32_t *topk_idx, *counts, *offsets, *perm, *inv_perm;
   float* topk_w;
   void *disp_ws, *router_ws, *xn, *xe, *h, *ye, *shared_h;
+  // W8A8: the token rows as block-scaled e4m3 (in the place of xe) and the gated product likewise
+  // (in the place of h)
+  void *xq, *xs, *hq, *hs;
   int64_t max_rows, disp_ws_bytes, router_ws_bytes, total;
 };
 
 ForwardBuffers carve_forward(void* workspace, int32_t T, int32_t D, int32_t E, int32_t K, int32_t F,
                              int32_t F_shared, int32_t tile_m, int32_t act_dtype, bool need_xe,
-                             bool need_xn) {
+                             bool need_xn, bool act_q = false) {
   const int64_t esz = fs2moe::elem_size(act_dtype);
   ForwardBuffers b;
   b.max_rows = FS2MOE_MAX_ROWS(T, K, E, tile_m);
@@ -70,7 +73,19 @@ ForwardBuffers carve_forward(void* workspace, int32_t T, int32_t D, int32_t E, i
   b.router_ws = b.router_ws_bytes > 0 ? c.take(b.router_ws_bytes) : nullptr;
   b.xn = need_xn ? c.take((int64_t)T * D * esz) : nullptr;
   b.xe = need_xe ? c.take(b.max_rows * D * esz) : nullptr;
+  b.xq = b.xs = b.hq = b.hs = nullptr;
+  if (act_q) {
+    // T rows of D codes and D / 32 scale bytes each: less than the row copy that is not made, so a
+    // workspace of fs2moe_forward_workspace_bytes (sized with the copy) holds them
+    b.xq = c.take((int64_t)T * D);
+    b.xs = c.take((int64_t)T * (D / 32));
+  }
   b.h = c.take(b.max_rows * F * esz);
+  if (act_q) {
+    // max_rows x (F codes + F / 32 scale bytes) inside the bf16 product's place
+    b.hq = b.h;
+    b.hs = static_cast<uint8_t*>(b.h) + (b.max_rows * F + 255) / 256 * 256;
+  }
   b.ye = c.take(b.max_rows * D * esz);
   b.shared_h = F_shared > 0 ? c.take((int64_t)T * F_shared * esz) : nullptr;
   b.total = c.used;
@@ -107,6 +122,8 @@ int forward_impl(bool normed, const void* x_in, const void* norm_weight, float n
                  int32_t w_dtype, int32_t score_fn, int32_t renormalize, int32_t scale_input,
                  void* workspace, int64_t workspace_bytes, void* out, void* stream) {
   const void* x = x_in;
+  const bool act_q = (w_dtype & FS2MOE_ACT_MXFP8) != 0;
+  w_dtype &= ~FS2MOE_ACT_MXFP8;
   FS2_REQUIRE(x && router && w_gate && w_up && w_down && out, "forward: null pointer");
   FS2_REQUIRE(T >= 0 && D >= 1 && E >= 1 && K >= 1 && F >= 1 && F_shared >= 0 && tile_m >= 1,
               "forward: bad sizes T=%d D=%d E=%d K=%d F=%d F_shared=%d tile_m=%d", T, D, E, K, F,
@@ -132,8 +149,18 @@ int forward_impl(bool normed, const void* x_in, const void* norm_weight, float n
   const int64_t widest = (int64_t)FS2MOE_MAX_ROWS(T, K, E, tile_m) * (D > F ? D : F) * 2;
   const bool fused = !scale_input && fs2moe_grouped_swiglu_fuses_gather(D, F, act_dtype, w_dtype) &&
                      (w_dtype == FS2MOE_FP8_E4M3 || widest <= 0xffffffffll);
+  if (act_q) {
+    FS2_REQUIRE(w_dtype == FS2MOE_FP8_E4M3 && act_dtype == FS2MOE_BF16 && s_gate && s_up && s_down,
+                "forward: FS2MOE_ACT_MXFP8 goes with e4m3 weights, their scales and bf16 rows");
+    FS2_REQUIRE(!scale_input, "forward: FS2MOE_ACT_MXFP8 with scale_input is not built into this "
+                              "call; use the stage calls");
+    FS2_REQUIRE(fs2moe_grouped_swiglu_w8a8_supported(D, F, FS2MOE_MAX_ROWS(T, K, E, tile_m)),
+                "forward: FS2MOE_ACT_MXFP8 with D=%d, F=%d: sizes the W8A8 kernels do not take "
+                "(fs2moe_grouped_swiglu_w8a8_supported)", D, F);
+  }
   const ForwardBuffers b = carve_forward(workspace, T, D, E, K, F, shared ? F_shared : 0, tile_m,
-                                         act_dtype, !fused, normed);
+                                         act_dtype, !fused && !act_q, normed, act_q);
+  FS2_REQUIRE(b.total <= need, "forward: internal: the W8A8 buffers do not fit the workspace");
   // (with a few tokens and no rows to copy the router's kernel dispatches as well)
   fs2moe::DispatchAfterRouter disp = {tile_m, b.max_rows, b.counts, b.offsets, b.perm, b.inv_perm, false};
   if (int rc = fs2moe::router_then_dispatch(x, normed ? norm_weight : nullptr, normed ? norm_eps : 0.f,
@@ -148,6 +175,14 @@ int forward_impl(bool normed, const void* x_in, const void* norm_weight, float n
                                  scale_input, b.max_rows, b.counts, b.offsets, b.perm, b.inv_perm,
                                  b.xe, b.disp_ws, b.disp_ws_bytes, stream))
       return rc;
+  if (act_q) {
+    // the token rows to block-scaled e4m3 once; both products read codes (the first through perm)
+    if (int rc = fs2moe_mx_quantize(x, T, D, b.xq, b.xs, stream)) return rc;
+    if (int rc = fs2moe_grouped_swiglu_w8a8(b.xq, b.xs, b.perm, b.counts, b.offsets, w_gate, w_up,
+                                            w_down, s_gate, s_up, s_down, E, D, F, T, b.max_rows,
+                                            b.hq, b.hs, b.ye, stream))
+      return rc;
+  } else
   // (a token takes an expert at most once: with up to 16 tokens no expert has more rows than that)
   if (int rc = fs2moe_grouped_swiglu_rows(fused ? x : b.xe, fused ? b.perm : nullptr, b.counts,
                                           b.offsets, w_gate, w_up, w_down, s_gate, s_up, s_down, E,

@@ -526,9 +526,12 @@ class MoE(FeedForwardNetwork):
         ex, se = self.experts, self.shared_expert
         w8a8 = type(ex) is GroupedExpertNetwork and ex.runs_w8a8(
             x.dtype, x.shape[0] * self.top_k + ex.num_local_experts * (self.tile_m - 1))
-        if (type(ex) is GroupedExpertNetwork and ex.has_fused_gate and not w8a8
+        # (W8A8 inside the one call wherever the call takes it: output-side weights, not under a
+        # compiler's trace, whose registered operator does not carry the option)
+        w8a8_staged = w8a8 and (self.scale_on == "input" or torch.compiler.is_compiling())
+        if (type(ex) is GroupedExpertNetwork and ex.has_fused_gate and not w8a8_staged
                 and (se is None or type(se) is GLUFeedForwardNetwork)):
-            return self._single_call(x, res, norm_args).view(seqs.shape)
+            return self._single_call(x, res, norm_args, act_quant=w8a8).view(seqs.shape)
         if wants_grad:
             # (only reachable inside a compiler's trace: the staged path below records no graph)
             raise RuntimeError(
@@ -618,7 +621,8 @@ class MoE(FeedForwardNetwork):
         """The router matrix expert-major (see :func:`fairseq2_amd._abi.router_expert_major`)."""
         return _abi.router_expert_major(self.router, self)
 
-    def _single_call(self, x: Tensor, residual: Tensor | None = None, norm=None) -> Tensor:
+    def _single_call(self, x: Tensor, residual: Tensor | None = None, norm=None, *,
+                     act_quant: bool = False) -> Tensor:
         """The layer through the library's whole-layer entry point: one call, one workspace
         allocation (same kernels and results as :meth:`_stages`)."""
         ex, se = self.experts, self.shared_expert
@@ -650,7 +654,7 @@ class MoE(FeedForwardNetwork):
             x, self.router.detach(), self.router_bias, *weights, ex.num_local_experts, self.top_k,
             scales=scales, shared=shared, tile_m=self.tile_m, score_fn=_SCORE_FNS[self.score_fn],
             renormalize=self.renormalize, scale_input=self.scale_on == "input", residual=residual,
-            norm=norm, router_t=self._router_expert_major(),
+            norm=norm, router_t=self._router_expert_major(), act_quant=act_quant,
         )
 
     @torch.no_grad()

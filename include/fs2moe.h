@@ -26,12 +26,18 @@
 extern "C" {
 #endif
 
-#define FS2MOE_ABI_VERSION 14
+#define FS2MOE_ABI_VERSION 15
 
 /* element types */
 #define FS2MOE_F32 0
 #define FS2MOE_BF16 1
 #define FS2MOE_FP8_E4M3 2 /* OCP e4m3fn codes, weights only, with per-output-channel f32 scales */
+/* May be OR-ed into the w_dtype argument of the whole-layer calls next to FS2MOE_FP8_E4M3: the expert
+ * products then run on the fp8 matrix pipe (W8A8), the rows rounded to block-scaled e4m3 on the way
+ * (fs2moe_mx_quantize, fs2moe_grouped_swiglu_w8a8 inside the call; an opt-in with no counterpart in
+ * the reference).  Accepted for bf16 activations, scale_input 0 and sizes for which
+ * fs2moe_grouped_swiglu_w8a8_supported(D, F, FS2MOE_MAX_ROWS(T, K, E, tile_m)) returns 1. */
+#define FS2MOE_ACT_MXFP8 0x100
 
 /* router score functions */
 #define FS2MOE_SCORE_SIGMOID 0 /* reference: sigmoid of the selected raw logit (moe.py:113,127) */
@@ -230,7 +236,9 @@ int fs2moe_combine_residual(const void* ye, const int32_t* inv_perm, const int32
  * itself; the result is what the five calls above give, bit for bit (they are what it calls).
  *   x [T, D] act_dtype            router [D, E] act_dtype          router_bias [E] f32 or NULL
  *   residual [T, D] act_dtype or NULL: added to the output as in fs2moe_combine_residual
- *   w_gate, w_up, w_down, s_*     as for fs2moe_grouped_swiglu
+ *   w_gate, w_up, w_down, s_*     as for fs2moe_grouped_swiglu; w_dtype FS2MOE_FP8_E4M3 | FS2MOE_ACT_MXFP8
+ *               runs the experts as fs2moe_grouped_swiglu_w8a8 does (the quantised rows take the
+ *               place of the row copy in the workspace, whose size does not change)
  *   shared_gate, shared_up [F_shared, D], shared_down [D, F_shared] act_dtype, or all NULL
  *   scale_input 1: combine weights multiply the experts' input rows (the reference, moe.py:132-134);
  *               0: they multiply the experts' output rows

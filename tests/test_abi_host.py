@@ -40,13 +40,19 @@ def test_library_exports_every_declared_symbol(lib):
 
 
 def test_abi_version_and_limits(lib):
-    assert lib.fs2moe_abi_version() == _abi.ABI_VERSION == 14
+    assert lib.fs2moe_abi_version() == _abi.ABI_VERSION == 15
     assert re.search(rf"#define FS2MOE_ABI_VERSION {_abi.ABI_VERSION}\b", open(HEADER).read())
     text = open(HEADER).read()
     assert f"#define FS2MOE_MAX_EXPERTS {_abi.MAX_EXPERTS}" in text
     assert f"#define FS2MOE_MAX_TOP_K {_abi.MAX_TOP_K}" in text
     for name, val in (("FS2MOE_F32", _abi.F32), ("FS2MOE_BF16", _abi.BF16), ("FS2MOE_FP8_E4M3", _abi.FP8_E4M3)):
         assert re.search(rf"#define {name} {val}\b", text)
+
+
+def test_header_and_wrapper_agree_on_the_w8a8_option():
+    assert re.search(rf"#define FS2MOE_ACT_MXFP8 {hex(_abi.ACT_MXFP8)}\b", open(HEADER).read())
+    # the option shares no bit with an element type
+    assert _abi.ACT_MXFP8 & (_abi.F32 | _abi.BF16 | _abi.FP8_E4M3) == 0
 
 
 def test_expert_major_router_is_taken_where_the_library_says_so(lib):

@@ -169,3 +169,47 @@ def test_qwen3_prefill_shape_w8a8(gpu_device):
     rel = float((got.double().cpu() - plain.double()).norm() / plain.double().norm())
     _say(f"  error against unquantised activations: {rel:.3%} of the norm")
     assert rel < 8e-2
+
+
+class _Norm:
+    def __init__(self, weight, eps):
+        self.weight, self.eps, self.normalized_shape = weight, eps, (weight.numel(),)
+
+
+def test_one_call_takes_the_fp8_pipe_and_equals_the_stages(gpu_device):
+    """``FS2MOE_ACT_MXFP8`` in the whole-layer call: the module's one call (with the normalisation
+    and the residual of a pre-norm decoder layer) against the same stages strung together, bit for
+    bit, and the refusals of the C entry point."""
+    _say("w8a8 one call")
+    spec = W.small_spec(tokens=900, model_dim=256, num_experts=8, top_k=2, inner_dim=128, dtype="bf16",
+                        weight_dtype="fp8", zipf_s=1.1, shared=True, mode=W.RoutingMode("softmax", True, "output"),
+                        seed=5, act_quant="mxfp8")
+    wl = W.make_workload_from_spec(spec)
+    m = build_module(wl, gpu_device)
+    g = torch.Generator().manual_seed(3)
+    raw = (1.7 * torch.randn(900, 256, generator=g)).to(torch.bfloat16).to(gpu_device)
+    gamma = (1.0 + 0.1 * torch.randn(256, generator=g)).to(torch.bfloat16).to(gpu_device)
+    norm = _Norm(gamma, 1e-5)
+    assert m.experts.runs_w8a8(torch.bfloat16, 900 * 2)
+    with torch.no_grad():
+        for residual, nrm in ((None, None), (raw, None), (raw, norm)):
+            got = m(raw, residual=residual, norm=nrm)
+            args = (raw, residual, None if nrm is None else (nrm.weight, nrm.eps))
+            assert torch.equal(got, m._single_call(*args, act_quant=True))
+            assert torch.equal(got, m._stages(*args)[0]), "the one call and the stages differ"
+            w8a16 = m._single_call(*args, act_quant=False)
+            assert not torch.equal(got, w8a16), "the option changed nothing"
+            rel = float((got.double() - w8a16.double()).norm() / w8a16.double().norm())
+            assert rel < 8e-2, rel
+    torch.cuda.synchronize()
+    # the C entry point refuses the option where it does not apply
+    ex = m.experts
+    weights = (ex.gate_q, ex.inner_q, ex.output_q)
+    scales = (ex.gate_scale, ex.inner_scale, ex.output_scale)
+    common = dict(scales=scales, score_fn=_abi.SCORE_SOFTMAX, renormalize=True)
+    with pytest.raises(RuntimeError, match="scale_input"):
+        _abi.forward(raw, m.router.detach(), m.router_bias, *weights, 8, 2, scale_input=True, act_quant=True, **common)
+    with pytest.raises(ValueError, match="e4m3"):
+        _abi.forward(raw, m.router.detach(), m.router_bias, ex.gate_proj.detach(), ex.inner_proj.detach(),
+                     ex.output_proj.detach(), 8, 2, scale_input=False, act_quant=True,
+                     score_fn=_abi.SCORE_SOFTMAX, renormalize=True)
