@@ -20,23 +20,25 @@
 // and two 32 x 256 weight sub-stages, 64 KB in all, and LDS holds two units.  The units of all of a
 // block's tiles form ONE stream: loads run ahead of the MFMAs straight across tile boundaries, so a
 // tile's epilogue overlaps the next tile's first loads.  A unit travels global -> registers -> LDS:
-//     producer, unit u:  barrier;  write unit u+1 from registers into the other half (read last in
-//                        unit u-1);  start loading unit u+2 into the registers
+//     producer, unit u:  barrier;  register by register: write the piece of unit u+1 it holds into
+//                        the other half (read last in unit u-1), load unit u+2's piece into it
 //     consumer, unit u:  barrier;  fragments from half u % 2;  32 MFMAs
 // One barrier per 64 k rather than per 32 k: after a barrier every consumer starts with LDS reads
 // whose latency nothing hides (both waves of a SIMD are at the same point), and that cost is per
-// barrier.  (Direct global->LDS loads would save the registers and the LDS writes, but a wave keeps
-// only two of them in flight, which caps four producers at 24 bytes per cycle; loads into distinct
-// registers are not limited that way and reach about three times that.)
+// barrier.  (Direct global->LDS loads would save the registers and the LDS writes, but in this
+// kernel four producers get 24 bytes per cycle out of them; loads into registers reach about three
+// times that.)
 //
-// What bounds it.  LDS traffic: a unit needs 64 KB stored (the four producers store at about
-// 50 B/clk while the consumers read) and 192 KB read (an activation block by 2 consumers, a weight
-// sub-tile by 4) inside the 2048 clocks of its MFMAs.  Measured in the kernel: the producers never
-// wait for memory once a second register set keeps two units in flight, yet spend half their time in
-// the 16 LDS stores of a unit; with all operands cache-resident the kernel is 7 % faster, with the
-// activation stores removed 11 %.  Per-wave LDS progress counters instead of the block barrier, a
-// second register set, and 128-k units for tiles of a few rows were each tried and each changed the
-// time by a few percent at most, so the simpler barrier per unit stayed.
+// What bounds it.  Per unit two chains of about the same length meet at the barrier: the consumers'
+// 2048 clocks of MFMAs, and a producer's 16 LDS stores (a 1 KB ds_write_b128 takes a wave about 80
+// clocks while the consumers read: 4 x 1 KB / 80 = 51 B/clk) and 16 loads (about 40 clocks each),
+// which as two phases took 1659 + 627 clocks and interleaved take about 2050; around the barrier
+// another 700 go by (the consumers' first fragment reads, the spread of twelve waves' arrival).
+// Measured and not kept, each within a few percent either way: a second register set (two units in
+// flight), per-wave LDS progress counters instead of the block barrier, direct global -> LDS loads
+// (about 170 clocks to issue each in this kernel), units of 128 k or two units in flight for tiles
+// of a few rows, consumer waves of 128 x 64, hand-pipelined and assembly consumer loops.  Under it
+// all the clock: the part holds 1.7-1.9 GHz with these operands, 2.4 with all-zero ones.
 //
 // LDS layout.  A wave writes its piece as one contiguous 1 KB, so rows are not padded; bank
 // conflicts are avoided by choosing WHICH global chunk each lane fetches (an XOR swizzle of the
