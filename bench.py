@@ -38,9 +38,9 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "mixtral_8x7b": 13.402e9,     # gate/up 8792 + 470 MB, down 4006 + 134 MB
     "llama4_scout": 6.677e9,      # routed experts only: gate/up 4103 + 135 MB, down 2355 + 84 MB
     "small_fp32": 0.866e9,        # gate/up 402 + 46 MB, down 401 + 17 MB
-    "qwen3_decode_fp8": 0.221e9,  # gate/up 143 + 1 MB, down 76 + 2 MB
+    "qwen3_decode_fp8": 0.222e9,  # gate/up 143 + 1 MB, down 76 + 2 MB
     "qwen3_30b_a3b_fp8": 1.886e9,  # gate/up 1033 + 101 MB, down 484 + 269 MB
-    "qwen3_30b_a3b_w8a8": 1.474e9,  # gate/up 777 + 67 MB, down 362 + 269 MB
+    "qwen3_30b_a3b_w8a8": 1.475e9,  # gate/up 778 + 67 MB, down 362 + 269 MB
 }
 
 
