@@ -443,16 +443,21 @@ __global__ __launch_bounds__(mx::NWAVES * 64) void glu_gemm_mx_kernel(
           const int X = block_exponent(amax);
           const float inv = __builtin_ldexpf(1.0f, -X);
           sbytes |= (uint32_t)(X + 127) << (8 * fn);
+          // (rows of 64 bytes: the 16-byte chunk index is XOR-ed with bits 2..3 of the row, or the 32
+          // lanes of a store, 64 bytes apart, would share four banks)
 #pragma unroll
-          for (int qq = 0; qq < 4; ++qq)
-            *reinterpret_cast<uint32_t*>(buf + lr * 64 + (8 * fn + 2 * qq + lk) * 4) =
+          for (int qq = 0; qq < 4; ++qq) {
+            const int dw = 8 * fn + 2 * qq + lk;  // dword of the row: chunk dw / 4
+            *reinterpret_cast<uint32_t*>(buf + lr * 64 + ((((dw >> 2) ^ (lr >> 2)) & 3) << 4) + (dw & 3) * 4) =
                 to_e4m3x4(v[4 * qq], v[4 * qq + 1], v[4 * qq + 2], v[4 * qq + 3], inv);
+          }
         }
         const int r0 = m_wave + fm * 32;
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
           const int rl = it * 16 + (lane >> 2);
-          const u32x4 val = *reinterpret_cast<const u32x4*>(buf + rl * 64 + (lane & 3) * 16);
+          const u32x4 val =
+              *reinterpret_cast<const u32x4*>(buf + rl * 64 + ((((lane & 3) ^ (rl >> 2)) & 3) << 4));
           if (col_ok && r0 + rl < t.row_end)
             __builtin_nontemporal_store(
                 val, reinterpret_cast<u32x4*>(C + (size_t)(r0 + rl) * ldc + n + (lane & 3) * 16));
