@@ -571,6 +571,61 @@ def test_dense_swiglu_matches_oracle(gpu_device, dtype, t, d, f):
     assert_output_close(y, ref, dtype, "shared expert")
 
 
+@pytest.mark.parametrize(
+    "rows,d,f,experts",
+    [
+        # tiles of 256 rows x 256 channels on 256 blocks.  Down projection (1 channel tile): 258 row
+        # tiles, the last of 208 rows: the two left over by the one whole round go out as halves,
+        # the second half of the last one 80 rows; gate/up (2 channel tiles): 516 tiles, 4 left over
+        (66000, 256, 256, 1),
+        # two experts of 198 + 99 row tiles (the last of each partly filled): 41 left over, as halves
+        (76000, 256, 128, 2),
+        # 384 + 1 tiles: 129 left over would be 258 halves, one too many: dealt whole
+        (98560, 256, 128, 1),
+    ],
+)
+def test_tiles_around_the_last_round_of_the_deal(gpu_device, rows, d, f, experts):
+    """The throughput kernel deals its tiles round-robin to one block per CU and splits the heavy
+    tiles that do not fill a round into halves when they then fit one round: shapes on both sides of
+    that rule, the grouped experts reading their rows through a map and the dense network, checked
+    on sampled rows (every row depends on its own tile only)."""
+    _say("last round of the deal", rows, d, f, experts)
+    g = torch.Generator().manual_seed(rows)
+    dev = gpu_device
+    tokens = 4096
+    x = torch.randn(tokens, d, generator=g).to(torch.bfloat16)
+    row_map = torch.randint(0, tokens, (rows,), generator=g, dtype=torch.int32)
+    first = rows * 2 // 3 if experts == 2 else rows
+    counts = torch.tensor([first, rows - first][:experts], dtype=torch.int32)
+    offsets = torch.tensor([0, first, rows][: experts + 1], dtype=torch.int32)
+    wg, wu = (0.05 * torch.randn(experts * d, f, generator=g) for _ in range(2))
+    wd = 0.05 * torch.randn(experts * f, d, generator=g)
+    wg, wu, wd = (w.to(torch.bfloat16) for w in (wg, wu, wd))
+    ye, _ = _abi.grouped_swiglu(x.to(dev), counts.to(dev), offsets.to(dev), wg.to(dev), wu.to(dev), wd.to(dev),
+                                experts, row_map=row_map.to(dev))
+    torch.cuda.synchronize()
+    # the first and last rows of every tile boundary region, and a random sample
+    pick = torch.cat([torch.arange(0, 3), torch.arange(rows - 400, rows), torch.arange(first - 200, min(first + 200, rows)),
+                      torch.randint(0, rows, (300,), generator=g)]).unique()
+    got = ye[pick.to(dev)]
+    for e in range(experts):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        sel = (pick >= lo) & (pick < hi)
+        if not bool(sel.any()):
+            continue
+        xr = x[row_map[pick[sel]].long()].double()
+        ref = O.glu_expert(xr, wg[e * d : (e + 1) * d].double(), wu[e * d : (e + 1) * d].double(),
+                           wd[e * f : (e + 1) * f].double())
+        assert_output_close(got[sel.to(dev)], ref, "bf16", f"expert {e}")
+    if experts == 1:
+        # the same rows through the dense network (nn.Linear-oriented weights, no map)
+        xs = x[row_map.long()].contiguous()
+        y = _abi.dense_swiglu(xs.to(dev), wg.t().contiguous().to(dev), wu.t().contiguous().to(dev),
+                              wd.t().contiguous().to(dev))
+        ref = O.shared_glu(xs[pick].double(), wg.t().double(), wu.t().double(), wd.t().double())
+        assert_output_close(y[pick.to(dev)], ref, "bf16", "dense network")
+
+
 # ----------------------------------------------------------------------------------------- combine
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
 @pytest.mark.parametrize("weight_output", [False, True])
