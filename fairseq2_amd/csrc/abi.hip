@@ -162,7 +162,8 @@ int forward_impl(bool normed, const void* x_in, const void* norm_weight, float n
                                          act_dtype, !fused && !act_q, normed, act_q);
   FS2_REQUIRE(b.total <= need, "forward: internal: the W8A8 buffers do not fit the workspace");
   // (with a few tokens and no rows to copy the router's kernel dispatches as well)
-  fs2moe::DispatchAfterRouter disp = {tile_m, b.max_rows, b.counts, b.offsets, b.perm, b.inv_perm, false};
+  fs2moe::DispatchAfterRouter disp = {tile_m,     b.max_rows, b.counts,        b.offsets, b.perm,
+                                      b.inv_perm, b.disp_ws,  b.disp_ws_bytes, false};
   if (int rc = fs2moe::router_then_dispatch(x, normed ? norm_weight : nullptr, normed ? norm_eps : 0.f,
                                     normed ? b.xn : nullptr, router, router_bias, T, D, E, K,
                                     act_dtype, score_fn, renormalize, b.topk_idx, b.topk_w,

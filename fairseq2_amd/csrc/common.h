@@ -169,14 +169,35 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline int elem_size(int dtype) { return dtype == FS2MOE_F32 ? 4 : dtype == FS2MOE_BF16 ? 2 : 1; }
 
 // Where the whole-layer call wants its dispatch (no rows copied): with at most 32 bf16 tokens the
-// router's finishing kernel ends with it and sets `done`; at any other size the router leaves
-// `done` false and the caller runs fs2moe_dispatch.  Either way the arrays hold the same values.
+// router's finishing kernel ends with it, and where one block routes a whole tile of 32 tokens from an
+// (E, D) matrix (up to kIndexTilesMax tiles) that block also counts the tile's pairs per expert and
+// ranks them, which leaves one dispatch kernel to run (dispatch_index_tiles); both set `done`.  At
+// any other size the router leaves `done` false and the caller runs fs2moe_dispatch.  Either way the
+// arrays hold the same values.  `ws` is the dispatch workspace (fs2moe_dispatch_workspace_bytes).
 struct DispatchAfterRouter {
   int tile_m;
   int64_t max_rows;
   int32_t *counts, *offsets, *perm, *inv_perm;
+  void* ws;
+  int64_t ws_bytes;
   bool done;
 };
+constexpr int kRouterTileTok = 32;   // tokens per tile of the MFMA routers
+constexpr int kIndexTilesMax = 512;  // tiles whose counts every block of dispatch_index_tiles adds up
+// The dispatch workspace as the tile-counting router fills it: per tile and expert the number of the
+// tile's tokens that chose the expert (a byte: at most 32), then per pair its rank among the tile's
+// pairs of the same expert.
+inline uint8_t* tile_counts_of(void* ws) { return static_cast<uint8_t*>(ws); }
+inline int32_t* tile_rank_of(void* ws, int T, int E) {
+  const int64_t nt = (T + kRouterTileTok - 1) / kRouterTileTok;
+  return reinterpret_cast<int32_t*>(static_cast<uint8_t*>(ws) + (nt * E + 255) / 256 * 256);
+}
+// The rest of dispatch after such a router: offsets, counts, perm and inv_perm as fs2moe_dispatch
+// writes them without a row copy.  E a multiple of 8, at most 256; at most kIndexTilesMax tiles.
+int dispatch_index_tiles(const int32_t* topk_idx, int32_t T, int32_t K, int32_t E, int32_t tile_m,
+                         int64_t max_rows, const uint8_t* tile_counts, const int32_t* tile_rank,
+                         int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv_perm,
+                         void* stream);
 // fs2moe_router_topk (xn null) or fs2moe_router_topk_norm, without the logits output
 int router_then_dispatch(const void* x, const void* norm_w, float norm_eps, void* xn,
                          const void* router, const float* bias, int32_t T, int32_t D, int32_t E,

@@ -316,6 +316,116 @@ __global__ __launch_bounds__(256) void dispatch_index_scan_kernel(
   perm[row] = t;
 }
 
+// The index pass after a router that counted for itself: tile_counts[tile][e] (bytes) is the number
+// of tile `tile`'s 32 tokens that chose expert e and tile_rank[p] the rank of pair p among its
+// tile's pairs of the same expert, token-ascending.  Block b < tile_blocks places the pairs of tile b;
+// as in dispatch_index_scan_kernel every block adds the table up for itself (num_tiles x E bytes
+// from L2: thread (slice, group of 8 experts) takes every S-th tile, 8 bytes a load, all of a
+// round's loads issued before any is looked at), block 0 writes counts and offsets, and the blocks
+// past the tiles fill the padding rows of perm.  Same integers as the other dispatch kernels.
+// E a multiple of 8 and at most 256 (one thread per expert in the scan).
+constexpr int kTileSumLoads = 8;
+__global__ __launch_bounds__(256) void dispatch_index_tiles_kernel(
+    const int32_t* __restrict__ topk_idx, int T, int K, int E, int tile_m, int64_t max_rows,
+    unsigned tile_blocks, const uint8_t* __restrict__ tile_counts, int num_tiles,
+    const int32_t* __restrict__ tile_rank, int32_t* __restrict__ counts,
+    int32_t* __restrict__ offsets, int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm) {
+  __shared__ int32_t s_part[2][2048];  // [all tiles | tiles before mine][slice][expert]: S E <= 2048
+  __shared__ int32_t s_off[257], s_cnt[256], s_pre[256];
+  __shared__ int32_t s_wave_tot[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const bool tile_block = blockIdx.x < tile_blocks;
+  const int mine = tile_block ? (int)blockIdx.x : 0;
+  const int G = E >> 3, S = 256 / G;
+  const int g = tid % G, sl = tid / G;
+  if (sl < S) {
+    int tot[8], pre[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) tot[j] = pre[j] = 0;
+    for (int t0 = sl; t0 < num_tiles; t0 += S * kTileSumLoads) {
+      uint2 c[kTileSumLoads];
+#pragma unroll
+      for (int i = 0; i < kTileSumLoads; ++i) {
+        const int tile = t0 + i * S;
+        c[i] = *reinterpret_cast<const uint2*>(tile_counts + (size_t)(tile < num_tiles ? tile : 0) * E +
+                                               g * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < kTileSumLoads; ++i) {
+        const int tile = t0 + i * S;
+        const bool in = tile < num_tiles, before = tile < mine;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int v = in ? (int)(((j < 4 ? c[i].x : c[i].y) >> (8 * (j & 3))) & 0xffu) : 0;
+          tot[j] += v;
+          pre[j] += before ? v : 0;
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      s_part[0][sl * E + g * 8 + j] = tot[j];
+      s_part[1][sl * E + g * 8 + j] = pre[j];
+    }
+  }
+  __syncthreads();
+  int padded = 0;
+  if (tid < E) {
+    int run = 0, pre = 0;
+    for (int i = 0; i < S; ++i) {
+      run += s_part[0][i * E + tid];
+      pre += s_part[1][i * E + tid];
+    }
+    s_cnt[tid] = run;
+    s_pre[tid] = pre;
+    padded = (run + tile_m - 1) / tile_m * tile_m;
+  }
+  int incl = padded;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    int v = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += v;
+  }
+  if (lane == 63) s_wave_tot[wave] = incl;
+  __syncthreads();
+  int base = 0;
+  for (int w = 0; w < wave; ++w) base += s_wave_tot[w];
+  if (tid < E) s_off[tid] = base + incl - padded;
+  if (tid == E - 1) s_off[E] = base + incl;
+  __syncthreads();
+  if (blockIdx.x == 0) {
+    if (tid < E) {
+      counts[tid] = s_cnt[tid];
+      offsets[tid] = s_off[tid];
+    }
+    if (tid == 0) offsets[E] = s_off[E];
+  }
+  if (!tile_block) {
+    const int idx = blockIdx.x - tile_blocks;
+    if (idx < E) {
+      const int64_t lo = (int64_t)s_off[idx] + s_cnt[idx], hi = s_off[idx + 1];
+      for (int64_t r = lo + tid; r < hi; r += 256) perm[r] = -1;
+    } else {
+      const int64_t r = (int64_t)s_off[E] + (int64_t)(idx - E) * 256 + tid;
+      if (r < max_rows) perm[r] = -1;
+    }
+    return;
+  }
+  const int64_t p0 = (int64_t)mine * kRouterTileTok * K, pairs = (int64_t)T * K;
+  for (int i = tid; i < kRouterTileTok * K; i += 256) {
+    const int64_t p = p0 + i;
+    if (p >= pairs) break;
+    const int e = topk_idx[p];
+    if (e < 0 || e >= E) {
+      inv_perm[p] = -1;
+      continue;
+    }
+    const int row = s_off[e] + s_pre[e] + tile_rank[p];
+    inv_perm[p] = row;
+    perm[row] = (int)(p / K);
+  }
+}
+
 // All of dispatch for at most 256 tokens when no rows are copied (xe == NULL): count, scan and
 // index in one block.  A decode step spends more on starting three kernels than on their work.
 // Same arithmetic as the three kernels above, so the results are identical.
@@ -383,10 +493,31 @@ __global__ __launch_bounds__(kDispTok) void dispatch_small_copy_kernel(
 
 using namespace fs2moe;
 
+int fs2moe::dispatch_index_tiles(const int32_t* topk_idx, int32_t T, int32_t K, int32_t E,
+                                 int32_t tile_m, int64_t max_rows, const uint8_t* tile_counts,
+                                 const int32_t* tile_rank, int32_t* counts, int32_t* offsets,
+                                 int32_t* perm, int32_t* inv_perm, void* stream) {
+  const int nt = (T + kRouterTileTok - 1) / kRouterTileTok;
+  FS2_REQUIRE(E % 8 == 0 && E <= 256 && nt >= 1 && nt <= kIndexTilesMax,
+              "dispatch: internal: E=%d, %d tiles given to the tile form", E, nt);
+  FS2_REQUIRE(max_rows >= FS2MOE_MAX_ROWS(T, K, E, tile_m) && max_rows < (1ll << 31),
+              "dispatch: max_rows=%lld outside [%lld, 2^31)", (long long)max_rows,
+              (long long)FS2MOE_MAX_ROWS(T, K, E, tile_m));
+  const unsigned tail_blocks = (unsigned)((max_rows - (int64_t)T * K + 255) / 256);
+  hipLaunchKernelGGL(dispatch_index_tiles_kernel, dim3((unsigned)nt + (unsigned)E + tail_blocks),
+                     dim3(256), 0, static_cast<hipStream_t>(stream), topk_idx, T, K, E, tile_m,
+                     max_rows, (unsigned)nt, tile_counts, nt, tile_rank, counts, offsets, perm,
+                     inv_perm);
+  return check_launch("dispatch_index_tiles");
+}
+
 extern "C" int64_t fs2moe_dispatch_workspace_bytes(int32_t T, int32_t K, int32_t E) {
   if (T < 0 || K < 1 || E < 1) return -1;
   const int64_t nb = (T + kDispTok - 1) / kDispTok;
-  int64_t bytes = (nb * E + (int64_t)T * K) * (int64_t)sizeof(int32_t);
+  // per-block counts and per-pair ranks; twice the counts' room so that the same bytes also hold
+  // the form a tile-counting router leaves (a byte per expert and tile of 32 tokens, then the
+  // ranks from the next multiple of 256 bytes on: tile_rank_of)
+  int64_t bytes = (2 * nb * E + (int64_t)T * K) * (int64_t)sizeof(int32_t);
   return (bytes + 255) / 256 * 256 + 256;
 }
 

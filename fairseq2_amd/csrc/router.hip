@@ -33,7 +33,7 @@ template <int J>
 __device__ __forceinline__ void select_topk(const float (&v)[J], int lane, int t, int E, int K,
                                             int score_fn, int renorm,
                                             int32_t* __restrict__ topk_idx,
-                                            float* __restrict__ topk_w) {
+                                            float* __restrict__ topk_w, int* chosen = nullptr) {
   // Keys of real logits are at least order_key(-inf) = 0x007fffff, so 0 marks "taken / no expert".
   uint32_t key[J];
 #pragma unroll
@@ -91,6 +91,7 @@ __device__ __forceinline__ void select_topk(const float (&v)[J], int lane, int t
     topk_idx[(size_t)t * K + lane] = my_e;
     topk_w[(size_t)t * K + lane] = w;
   }
+  if (chosen != nullptr) *chosen = my_e;  // lane r < K: the token's r-th expert
 }
 
 // ------------------------------------------------------------------------------------- f32 / FMA
@@ -607,7 +608,7 @@ __global__ __launch_bounds__(1024) void router_mfma_t_kernel(
     const uint16_t* x, const uint16_t* norm_w, float norm_eps, uint16_t* xn,
     const uint16_t* __restrict__ router_t, const float* __restrict__ bias, int T, int D, int E, int K,
     int score_fn, int renorm, int32_t* __restrict__ topk_idx, float* __restrict__ topk_w,
-    float* __restrict__ logits) {
+    float* __restrict__ logits, uint8_t* __restrict__ tile_counts, int32_t* __restrict__ tile_rank) {
   using namespace rmfma_t;
   using S = Shape<NF>;
   constexpr int EP = S::EP, LDL = S::LDL, SLOTS = S::SLOTS, AHEAD = SLOTS - 1, J = EP / 64, TPS = S::TPS;
@@ -726,25 +727,48 @@ __global__ __launch_bounds__(1024) void router_mfma_t_kernel(
       f32x4 v = {acc[f][4 * q], acc[f][4 * q + 1], acc[f][4 * q + 2], acc[f][4 * q + 3]};
       *reinterpret_cast<f32x4*>(&sL[lr * LDL + e]) = v;
     }
+  // With tile_counts the block also does the counting pass of dispatch for its 32 tokens: a word
+  // per expert, bit `token of the tile` set by the lane that holds the choice (an order-independent
+  // OR), from which a pair's rank among the tile's pairs of its expert is a population count.
+  static_assert(S::LOGIT_BYTES + EP * 4 <= S::SMEM_BYTES, "room for the tile's membership words");
+  uint32_t* s_bits = reinterpret_cast<uint32_t*>(smem_t + S::LOGIT_BYTES);
+  const bool counting = tile_counts != nullptr;  // block-uniform
+  if (counting && tid < EP) s_bits[tid] = 0u;
   __syncthreads();
 
   constexpr int TPW = BT / 16;  // every wave selects for two tokens
+  int chosen[TPW];
+#pragma unroll
   for (int i = 0; i < TPW; ++i) {
     const int tl = wave * TPW + i;
     const int t = t0 + tl;
-    if (t >= T) break;  // wave-uniform
-    float v[J];
+    chosen[i] = 0;
+    if (t < T) {  // wave-uniform
+      float v[J];
 #pragma unroll
-    for (int j = 0; j < J; ++j) {
-      const int e = lane + 64 * j;
-      float sum = 0.f;
+      for (int j = 0; j < J; ++j) {
+        const int e = lane + 64 * j;
+        float sum = 0.f;
 #pragma unroll
-      for (int g2 = 0; g2 < 4; ++g2) sum += reinterpret_cast<const float*>(smem_t)[g2 * (BT * LDL) + tl * LDL + e];
-      v[j] = sum + b[j];
-      if (logits != nullptr && e < E) logits[(size_t)t * E + e] = v[j];
+        for (int g2 = 0; g2 < 4; ++g2)
+          sum += reinterpret_cast<const float*>(smem_t)[g2 * (BT * LDL) + tl * LDL + e];
+        v[j] = sum + b[j];
+        if (logits != nullptr && e < E) logits[(size_t)t * E + e] = v[j];
+      }
+      select_topk<J>(v, lane, t, E, K, score_fn, renorm, topk_idx, topk_w, &chosen[i]);
+      if (counting && lane < K) atomicOr(&s_bits[chosen[i]], 1u << tl);
     }
-    select_topk<J>(v, lane, t, E, K, score_fn, renorm, topk_idx, topk_w);
   }
+  if (!counting) return;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < TPW; ++i) {
+    const int tl = wave * TPW + i;
+    const int t = t0 + tl;
+    if (t < T && lane < K)
+      tile_rank[(size_t)t * K + lane] = __popc(s_bits[chosen[i]] & ((1u << tl) - 1u));
+  }
+  if (tid < E) tile_counts[(size_t)blockIdx.x * E + tid] = (uint8_t)__popc(s_bits[tid]);
 }
 
 constexpr int kMaxSlices = 8;  // blocks sharing a token tile, at most
@@ -1142,15 +1166,29 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const uint16_t* wp = static_cast<const uint16_t*>(norm_w);
     uint16_t* xnp = static_cast<uint16_t*>(xn);
+    // (the whole-layer call without a row copy: the tiles count their pairs themselves)
+    static_assert(rmfma_t::BT == kRouterTileTok, "one routing block per counting tile");
+    const bool counting = disp != nullptr && disp->ws != nullptr && (int)grid.x <= kIndexTilesMax &&
+                          disp->ws_bytes >= fs2moe_dispatch_workspace_bytes(T, K, E);
+    uint8_t* tile_counts = counting ? tile_counts_of(disp->ws) : nullptr;
+    int32_t* tile_rank = counting ? tile_rank_of(disp->ws, T, E) : nullptr;
     if (E <= 128)
       hipLaunchKernelGGL(k1, grid, threads, rmfma_t::Shape<1>::SMEM_BYTES, s, xp, wp, norm_eps, xnp,
                          static_cast<const uint16_t*>(router), bias, T, D, E, K, score_fn, renormalize,
-                         topk_idx, topk_w, logits);
+                         topk_idx, topk_w, logits, tile_counts, tile_rank);
     else
       hipLaunchKernelGGL(k2, grid, threads, rmfma_t::Shape<2>::SMEM_BYTES, s, xp, wp, norm_eps, xnp,
                          static_cast<const uint16_t*>(router), bias, T, D, E, K, score_fn, renormalize,
-                         topk_idx, topk_w, logits);
-    return check_launch("router_mfma (E, D)");
+                         topk_idx, topk_w, logits, tile_counts, tile_rank);
+    if (int rc = check_launch("router_mfma (E, D)")) return rc;
+    if (counting) {
+      if (int rc = dispatch_index_tiles(topk_idx, T, K, E, disp->tile_m, disp->max_rows, tile_counts,
+                                        tile_rank, disp->counts, disp->offsets, disp->perm,
+                                        disp->inv_perm, stream))
+        return rc;
+      disp->done = true;
+    }
+    return FS2MOE_OK;
   }
   if (act_dtype == FS2MOE_F32) {
     // The MFMA path moves 16-byte chunks (D and E multiples of 4, aligned bases) and holds up to

@@ -128,7 +128,8 @@ int fs2moe_cpu_router_select(const float* logits, int32_t T, int32_t E, int32_t 
                              int32_t renormalize, int32_t* topk_idx, float* topk_w);
 
 /*
- * Bytes of device scratch fs2moe_dispatch needs (per-block histograms and ranks).
+ * Bytes of device scratch fs2moe_dispatch needs (per-block histograms and ranks; the whole-layer
+ * calls use the same bytes for the histograms their router kernel writes per 32 tokens).
  */
 int64_t fs2moe_dispatch_workspace_bytes(int32_t T, int32_t K, int32_t E);
 

@@ -384,6 +384,65 @@ def test_single_call_entry_point_equals_the_module(gpu_device, dtype, weight_dty
     assert torch.equal(got, out.reshape(-1, 128))
 
 
+@pytest.mark.parametrize(
+    "tokens,e,k,tile_m",
+    [
+        (33, 8, 2, 16),       # two tiles, the second with one token
+        (300, 8, 2, 16),
+        (1000, 24, 1, 16),    # groups of 8 experts that do not divide the block's threads
+        (2500, 64, 8, 1),     # no padding rows at all
+        (4100, 256, 32, 8),   # the two-fragment router, 1024 pairs per tile
+        (16384, 16, 4, 16),   # the most tiles the tile form takes
+        (16385, 16, 4, 16),   # one more: the counting kernel's form again
+    ],
+)
+def test_single_call_dispatches_like_the_dispatch_call(gpu_device, tokens, e, k, tile_m):
+    """Inside ``fs2moe_forward`` the router of an (E, D) matrix counts and ranks its own tiles of 32
+    tokens and one more kernel finishes the dispatch: the selection, the counts, the offsets and
+    both permutations, read back from the head of the workspace, against ``fs2moe_router_topk`` +
+    ``fs2moe_dispatch``, integer for integer; and the layer's output against the stages'."""
+    _say("single call dispatch", tokens, e, k, tile_m)
+    d, f = 128, 64
+    g = torch.Generator().manual_seed(tokens + e)
+    x = torch.randn(tokens, d, generator=g).bfloat16().to(gpu_device)
+    router = (torch.randn(d, e, generator=g) * 0.3).bfloat16().to(gpu_device)
+    # a few experts that nobody chooses, and ties between neighbours
+    bias = torch.zeros(e)
+    bias[e // 2:: 5] = -30.0
+    bias = bias.to(gpu_device)
+    router[:, 1] = router[:, 0]
+    wg = (torch.randn(e * d, f, generator=g) * 0.1).bfloat16().to(gpu_device)
+    wu = (torch.randn(e * d, f, generator=g) * 0.1).bfloat16().to(gpu_device)
+    wd = (torch.randn(e * f, d, generator=g) * 0.1).bfloat16().to(gpu_device)
+    rt = router.t().contiguous()
+    lib = _abi.load()
+    assert lib.fs2moe_router_takes_out_in(tokens, d, e, _abi.BF16) == 1
+    ws = torch.zeros(lib.fs2moe_forward_workspace_bytes(tokens, d, e, k, f, 0, tile_m, _abi.BF16),
+                     dtype=torch.uint8, device=gpu_device)
+    out = _abi.forward(x, router, bias, wg, wu, wd, e, k, tile_m=tile_m, score_fn=_abi.SCORE_SOFTMAX,
+                       renormalize=True, scale_input=False, workspace=ws, router_t=rt)
+    idx, w, _ = _abi.router_topk(x, router, bias, k, _abi.SCORE_SOFTMAX, True, router_t=rt)
+    dsp = _abi.dispatch(idx, w, x, e, tile_m, False, gather=False)
+    torch.cuda.synchronize()
+    # the head of the workspace: T x K indices, T x K weights, E counts, E + 1 offsets, max_rows of
+    # perm, T x K of inv_perm, each from the next multiple of 256 bytes on
+    rows = _abi.max_rows(tokens, k, e, tile_m)
+    at = 0
+    parts = []
+    for n in (tokens * k, tokens * k, e, e + 1, rows, tokens * k):
+        parts.append(ws[at: at + 4 * n].view(torch.int32))
+        at += (4 * n + 255) // 256 * 256
+    assert torch.equal(parts[0].view(tokens, k), idx), "the selection (which also places the parts)"
+    assert torch.equal(parts[1].view(torch.float32).view(tokens, k), w)
+    assert torch.equal(parts[2], dsp.counts) and int(dsp.counts.sum()) == tokens * k
+    assert int((dsp.counts == 0).sum()) > 0 or e == 8
+    assert torch.equal(parts[3], dsp.offsets)
+    assert torch.equal(parts[5].view(tokens, k), dsp.inv_perm)
+    assert torch.equal(parts[4], dsp.perm)
+    ye, _ = _abi.grouped_swiglu(x, dsp.counts, dsp.offsets, wg, wu, wd, e, row_map=dsp.perm)
+    assert torch.equal(out, _abi.combine(ye, dsp.inv_perm, idx, w, None, True))
+
+
 def test_expert_major_copy_of_the_router_follows_the_parameter(gpu_device):
     """The derived (E, D) copy the bf16 router reads: made once, made again after an in-place update,
     after a move and for another tensor (also one that reuses a freed tensor's address), and kept
