@@ -25,7 +25,10 @@ TORCH_DTYPE = {"fp32": torch.float32, "bf16": torch.bfloat16}
 #   and the rows scaled on the way in (a fourth rounding per term), atol = 2 % sits AT the expected
 #   maximum (a seeded case did land at 1.03 of it).  Such cases, and only they, pass atol_scale = 2
 #   (4e-2 * rms, 10 sigma); everything else is held to 2e-2.  The overall statement, RMS_TOL = 1e-2,
-#   is the sharp one everywhere: 2.7 sigma-units above the emulation's 0.37 %.
+#   is the sharp one everywhere: 2.7 sigma-units above the emulation's 0.37 %.  About one drawn case
+#   in a thousand still has a single element at 1.0-1.1 of the element-wise bound with few terms
+#   (two cancelling expert rows under a heavy-tailed gated product); the seeded sweep settles
+#   those against emulate_device_rounding below instead of widening the bound.
 # fp32: rtol 1e-4, atol 1e-4 * rms, RMS_TOL 2e-5 (f32 MFMA accumulation order differs from the CPU's).
 TOL = {"bf16": (2e-2, 2e-2), "fp32": (1e-4, 1e-4)}
 RMS_TOL = {"bf16": 1e-2, "fp32": 2e-5}
@@ -52,6 +55,13 @@ def oracle_forward(wl: W.Workload, idx, tile_m: int, tokens=None, dtype=torch.fl
     )
 
 
+def output_bound(ref: torch.Tensor, dtype: str, atol_scale: float = 1.0) -> torch.Tensor:
+    """The element-wise bound of :func:`assert_output_close`: atol tied to rms(ref), plus rtol |ref|."""
+    rtol, atol_rel = TOL[dtype]
+    ref = ref.double()
+    return atol_rel * atol_scale * float(ref.pow(2).mean().sqrt()) + rtol * ref.abs()
+
+
 def assert_output_close(got: torch.Tensor, ref: torch.Tensor, dtype: str, what: str = "output",
                         atol_scale: float = 1.0):
     got = got.detach().double().cpu().reshape(ref.shape)
@@ -61,7 +71,7 @@ def assert_output_close(got: torch.Tensor, ref: torch.Tensor, dtype: str, what: 
     rms = float(ref.pow(2).mean().sqrt())
     atol = atol_rel * rms
     err = (got - ref).abs()
-    bound = atol + rtol * ref.abs()
+    bound = output_bound(ref, dtype, atol_scale)
     worst = float((err / bound).max()) if err.numel() else 0.0
     assert torch.isfinite(got).all(), f"{what}: non-finite values"
     assert worst <= 1.0, (

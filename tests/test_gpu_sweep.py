@@ -18,7 +18,8 @@ from fairseq2_amd import _abi
 import workloads as W
 from oracle import moe_oracle as O
 from tests._util import (
-    TORCH_DTYPE, assert_output_close, assert_routing_equal, build_module, oracle_forward, oracle_routing,
+    TORCH_DTYPE, assert_output_close, assert_routing_equal, build_module, emulate_device_rounding, oracle_forward,
+    oracle_routing, output_bound,
 )
 
 pytestmark = pytest.mark.gpu
@@ -127,7 +128,31 @@ def _check_routing(c, wl, x2d, m, gi, it):
     return dev_idx, separated
 
 
-@pytest.mark.parametrize("seed", [11, 12, 13])
+def _explained_by_the_rounding_points(wl, c, idx, gw, res_c, single, want, atol_scale, it):
+    """An element outside the element-wise bound is the kernel's doing or the number format's.  The
+    same arithmetic on the CPU, in f32 with a bf16 rounding wherever the device (and the reference
+    module run in bf16) rounds, tells which: a heavy-tailed gated product rounds with an absolute
+    error that a pair of cancelling terms does not shrink, and an output element can then sit at
+    1.0-1.1 of the bound in that evaluation as well (about one case in a thousand, all seen in the
+    mode that scales the rows on the way in).  Accepted only if the device agrees with that
+    evaluation everywhere, the elements over the bound are a handful, none beyond 1.25, and the
+    CPU evaluation is out (or at the edge) at each of them too.  bf16 cases without a shared
+    expert; anything else stays a failure."""
+    emu = emulate_device_rounding(wl, idx, gw.cpu(), residual=res_c).double().reshape(want.shape)
+    got = single.detach().double().cpu().reshape(want.shape)
+    bound = output_bound(want, c["dtype"], atol_scale)
+    over = (got - want).abs() > bound
+    assert_output_close(single, emu, c["dtype"], f"case {it}: against the CPU evaluation with the device's roundings")
+    assert int(over.sum()) <= max(1, over.numel() // 10000), f"case {it}: {int(over.sum())} elements over the bound"
+    assert float(((got - want).abs() / bound).max()) <= 1.25, f"case {it}: beyond what the roundings explain"
+    assert bool((((emu - want).abs() / bound)[over] >= 0.9).all()), (
+        f"case {it}: over the bound where the CPU evaluation with the same roundings is inside it")
+    print(f"  case {it}: {int(over.sum())} element(s) at up to {float(((got - want).abs() / bound).max()):.3f} of the "
+          "bound, as in the CPU evaluation with the device's rounding points", flush=True)
+
+
+# (seed 52 holds a case of the kind _explained_by_the_rounding_points is for)
+@pytest.mark.parametrize("seed", [11, 12, 13, 52])
 def test_seeded_sweep(gpu_device, seed):
     rng = random.Random(seed)
     near_ties = 0
@@ -149,7 +174,7 @@ def test_seeded_sweep(gpu_device, seed):
             res = res_c.to(gpu_device)
         with torch.no_grad():
             single = m(x, residual=res)
-            staged, gi, _, disp = m.forward_with_routing(x)
+            staged, gi, gw, disp = m.forward_with_routing(x)
             if res is not None:
                 staged = m._stages(x.reshape(-1, c["d"]), res.reshape(-1, c["d"]))[0].view(x.shape)
         torch.cuda.synchronize()
@@ -161,7 +186,13 @@ def test_seeded_sweep(gpu_device, seed):
         assert_routing_equal(gi, disp, ref.routing, f"case {it}")
         # many terms, each rounded a fourth time on the way in: see tests/_util.py
         many_roundings = c["k"] >= 8 and c["mode"].scale_on == "input"
-        assert_output_close(single, want, c["dtype"], f"case {it}", atol_scale=2.0 if many_roundings else 1.0)
+        atol_scale = 2.0 if many_roundings else 1.0
+        try:
+            assert_output_close(single, want, c["dtype"], f"case {it}", atol_scale=atol_scale)
+        except AssertionError:
+            if c["dtype"] != "bf16" or c["shared"]:
+                raise
+            _explained_by_the_rounding_points(wl, c, idx, gw, res_c, single, want, atol_scale, it)
         if random.Random(1000 * seed + it).random() < 0.35:
             _check_norm_in_front(m, c, dt, res, gpu_device, it)
     print(f"sweep seed={seed}: {len(cases)} cases, {near_ties} with near-ties resolved through the host mirror", flush=True)
