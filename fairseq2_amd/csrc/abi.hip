@@ -51,12 +51,14 @@ struct ForwardBuffers {
   // W8A8: the token rows as block-scaled e4m3 (in the place of xe) and the gated product likewise
   // (in the place of h)
   void *xq, *xs, *hq, *hs;
+  // a weight per expert row (in the place of xe) where the expert kernels scale the rows themselves
+  float* row_w;
   int64_t max_rows, disp_ws_bytes, router_ws_bytes, total;
 };
 
 ForwardBuffers carve_forward(void* workspace, int32_t T, int32_t D, int32_t E, int32_t K, int32_t F,
                              int32_t F_shared, int32_t tile_m, int32_t act_dtype, bool need_xe,
-                             bool need_xn, bool act_q = false) {
+                             bool need_xn, bool act_q = false, bool need_row_w = false) {
   const int64_t esz = fs2moe::elem_size(act_dtype);
   ForwardBuffers b;
   b.max_rows = FS2MOE_MAX_ROWS(T, K, E, tile_m);
@@ -73,6 +75,8 @@ ForwardBuffers carve_forward(void* workspace, int32_t T, int32_t D, int32_t E, i
   b.router_ws = b.router_ws_bytes > 0 ? c.take(b.router_ws_bytes) : nullptr;
   b.xn = need_xn ? c.take((int64_t)T * D * esz) : nullptr;
   b.xe = need_xe ? c.take(b.max_rows * D * esz) : nullptr;
+  // (4 bytes a row where the copy would have taken D elements: the workspace sized with the copy holds it)
+  b.row_w = need_row_w ? static_cast<float*>(c.take(b.max_rows * 4)) : nullptr;
   b.xq = b.xs = b.hq = b.hs = nullptr;
   if (act_q) {
     // T rows of D codes and D / 32 scale bytes each: less than the row copy that is not made, so a
@@ -158,12 +162,20 @@ int forward_impl(bool normed, const void* x_in, const void* norm_weight, float n
                 "forward: FS2MOE_ACT_MXFP8 with D=%d, F=%d: sizes the W8A8 kernels do not take "
                 "(fs2moe_grouped_swiglu_w8a8_supported)", D, F);
   }
+  // The reference's routing mode multiplies each row by its routing weight on the way in, which
+  // dispatch does as it copies the rows.  With at most 16 bf16 tokens (a decode step) the expert
+  // kernels stage a few rows in LDS and stream the weights past them: they take the row from x
+  // through perm and scale it there, so that no copy is made and dispatch can run inside the router's
+  // second kernel as in the other mode.
+  const bool scaled_stream = scale_input && !act_q && T <= 16 && D * 2 >= 4 &&
+                             fs2moe::swiglu_streams_rows(act_dtype, w_dtype, D, F, E, T);
   const ForwardBuffers b = carve_forward(workspace, T, D, E, K, F, shared ? F_shared : 0, tile_m,
-                                         act_dtype, !fused && !act_q, normed, act_q);
-  FS2_REQUIRE(b.total <= need, "forward: internal: the W8A8 buffers do not fit the workspace");
+                                         act_dtype, !fused && !act_q && !scaled_stream, normed, act_q,
+                                         scaled_stream);
+  FS2_REQUIRE(b.total <= need, "forward: internal: the buffers do not fit the workspace");
   // (with a few tokens and no rows to copy the router's kernel dispatches as well)
   fs2moe::DispatchAfterRouter disp = {tile_m,     b.max_rows, b.counts,        b.offsets, b.perm,
-                                      b.inv_perm, b.disp_ws,  b.disp_ws_bytes, false};
+                                      b.inv_perm, b.disp_ws,  b.disp_ws_bytes, b.row_w, false};
   if (int rc = fs2moe::router_then_dispatch(x, normed ? norm_weight : nullptr, normed ? norm_eps : 0.f,
                                     normed ? b.xn : nullptr, router, router_bias, T, D, E, K,
                                     act_dtype, score_fn, renormalize, b.topk_idx, b.topk_w,
@@ -171,17 +183,29 @@ int forward_impl(bool normed, const void* x_in, const void* norm_weight, float n
                                     stream))
     return rc;
   if (normed) x = b.xn;
-  if (!disp.done)
-    if (int rc = fs2moe_dispatch(b.topk_idx, b.topk_w, x, T, K, E, D, tile_m, act_dtype,
-                                 scale_input, b.max_rows, b.counts, b.offsets, b.perm, b.inv_perm,
-                                 b.xe, b.disp_ws, b.disp_ws_bytes, stream))
+  if (!disp.done) {
+    if (scaled_stream) {
+      if (int rc = fs2moe::dispatch_with_row_weights(b.topk_idx, b.topk_w, T, K, E, tile_m, b.max_rows,
+                                                     b.counts, b.offsets, b.perm, b.inv_perm, b.row_w,
+                                                     stream))
+        return rc;
+    } else if (int rc = fs2moe_dispatch(b.topk_idx, b.topk_w, x, T, K, E, D, tile_m, act_dtype,
+                                        scale_input, b.max_rows, b.counts, b.offsets, b.perm,
+                                        b.inv_perm, b.xe, b.disp_ws, b.disp_ws_bytes, stream)) {
       return rc;
+    }
+  }
   if (act_q) {
     // the token rows to block-scaled e4m3 once; both products read codes (the first through perm)
     if (int rc = fs2moe_mx_quantize(x, T, D, b.xq, b.xs, stream)) return rc;
     if (int rc = fs2moe_grouped_swiglu_w8a8(b.xq, b.xs, b.perm, b.counts, b.offsets, w_gate, w_up,
                                             w_down, s_gate, s_up, s_down, E, D, F, T, b.max_rows,
                                             b.hq, b.hs, b.ye, stream))
+      return rc;
+  } else if (scaled_stream) {
+    if (int rc = fs2moe::grouped_swiglu_scaled_rows(x, b.perm, b.row_w, b.counts, b.offsets, w_gate,
+                                                    w_up, w_down, E, D, F, b.max_rows, b.h, b.ye, T,
+                                                    stream))
       return rc;
   } else
   // (a token takes an expert at most once: with up to 16 tokens no expert has more rows than that)

@@ -38,6 +38,12 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   const f32x2_t v = {lo, hi};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+// Two bf16 values times an f32 weight, each product rounded to bf16: what dispatch stores when it
+// copies a row scaled by its routing weight, and what a kernel that scales the row on the way in
+// must compute to give the same bits.
+__device__ __forceinline__ uint32_t scale_bf16x2(uint32_t v, float w) {
+  return pack_bf16x2(__uint_as_float(v << 16) * w, __uint_as_float(v & 0xffff0000u) * w);
+}
 
 template <typename T>
 struct Elem;
@@ -180,6 +186,9 @@ struct DispatchAfterRouter {
   int32_t *counts, *offsets, *perm, *inv_perm;
   void* ws;
   int64_t ws_bytes;
+  // optional (bf16 decode sizes, rows scaled by the routing weight on their way into the experts
+  // instead of by a copy): per expert row the weight of its pair, written next to perm
+  float* row_w;
   bool done;
 };
 constexpr int kRouterTileTok = 32;   // tokens per tile of the MFMA routers
@@ -204,6 +213,24 @@ int router_then_dispatch(const void* x, const void* norm_w, float norm_eps, void
                          int32_t K, int32_t act_dtype, int32_t score_fn, int32_t renormalize,
                          int32_t* topk_idx, float* topk_w, void* workspace, int64_t workspace_bytes,
                          DispatchAfterRouter* disp, void* stream);
+
+// fs2moe_dispatch without a row copy that also writes row_w[row] = topk_w[pair] (see
+// DispatchAfterRouter): at most 256 tokens and 256 experts, K <= 16 or not.
+int dispatch_with_row_weights(const int32_t* topk_idx, const float* topk_w, int32_t T, int32_t K,
+                              int32_t E, int32_t tile_m, int64_t max_rows, int32_t* counts,
+                              int32_t* offsets, int32_t* perm, int32_t* inv_perm, float* row_w,
+                              void* stream);
+// Whether the grouped SwiGLU pair of these sizes runs on the kernels that stream the weights past a
+// few staged rows (at most rows_per_expert of any expert), which can scale each row by row_w as
+// they stage it; and that pair: fs2moe_grouped_swiglu_rows with rows read through row_map and
+// multiplied by row_w[row] (rounded to bf16, as dispatch's scaled copy rounds them).
+bool swiglu_streams_rows(int32_t act_dtype, int32_t w_dtype, int32_t D, int32_t F, int32_t E,
+                         int32_t rows_per_expert);
+int grouped_swiglu_scaled_rows(const void* x, const int32_t* row_map, const float* row_w,
+                               const int32_t* counts, const int32_t* offsets, const void* w_gate,
+                               const void* w_up, const void* w_down, int32_t E, int32_t D, int32_t F,
+                               int64_t max_rows, void* h, void* ye, int32_t rows_per_expert,
+                               void* stream);
 
 }  // namespace fs2moe
 

@@ -132,11 +132,7 @@ template <>
 __device__ __forceinline__ u32x4 scale_chunk<uint16_t>(u32x4 v, float w) {
   u32x4 o;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    float lo = __uint_as_float(v[i] << 16) * w;
-    float hi = __uint_as_float(v[i] & 0xffff0000u) * w;
-    o[i] = pack_bf16x2(lo, hi);
-  }
+  for (int i = 0; i < 4; ++i) o[i] = scale_bf16x2(v[i], w);
   return o;
 }
 
@@ -433,11 +429,11 @@ template <int KCAP>
 __global__ __launch_bounds__(kDispTok) void dispatch_small_kernel(
     const int32_t* __restrict__ topk_idx, int T, int K, int E, int tile_m, int64_t max_rows,
     int32_t* __restrict__ counts, int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
-    int32_t* __restrict__ inv_perm) {
+    int32_t* __restrict__ inv_perm, const float* __restrict__ topk_w, float* __restrict__ row_w) {
   extern __shared__ uint32_t s_mem[];
   __shared__ int32_t s_wave_tot[4];
   dispatch_small_block<KCAP>(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm, s_mem,
-                       s_wave_tot, threadIdx.x, kDispTok);
+                       s_wave_tot, threadIdx.x, kDispTok, true, topk_w, row_w);
 }
 
 // All of dispatch for at most 256 tokens WITH the row copy, in one launch: every block works out the
@@ -511,6 +507,30 @@ int fs2moe::dispatch_index_tiles(const int32_t* topk_idx, int32_t T, int32_t K, 
   return check_launch("dispatch_index_tiles");
 }
 
+int fs2moe::dispatch_with_row_weights(const int32_t* topk_idx, const float* topk_w, int32_t T,
+                                      int32_t K, int32_t E, int32_t tile_m, int64_t max_rows,
+                                      int32_t* counts, int32_t* offsets, int32_t* perm,
+                                      int32_t* inv_perm, float* row_w, void* stream) {
+  FS2_REQUIRE(topk_idx && topk_w && counts && offsets && perm && inv_perm && row_w,
+              "dispatch: null pointer");
+  FS2_REQUIRE(T >= 1 && T <= kDispTok && E >= 1 && E <= kDispTok && K >= 1 && K <= FS2MOE_MAX_TOP_K,
+              "dispatch: internal: T=%d E=%d K=%d given to the one-block form", T, E, K);
+  FS2_REQUIRE(tile_m >= 1 && tile_m <= 1024, "dispatch: tile_m=%d", tile_m);
+  FS2_REQUIRE(max_rows >= FS2MOE_MAX_ROWS(T, K, E, tile_m) && max_rows < (1ll << 31),
+              "dispatch: max_rows=%lld outside [%lld, 2^31)", (long long)max_rows,
+              (long long)FS2MOE_MAX_ROWS(T, K, E, tile_m));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t lds = dispatch_small_lds_words(E) * sizeof(uint32_t);
+  if (K <= 16)
+    hipLaunchKernelGGL(dispatch_small_kernel<16>, dim3(1), dim3(kDispTok), lds, s, topk_idx, T, K, E,
+                       tile_m, max_rows, counts, offsets, perm, inv_perm, topk_w, row_w);
+  else
+    hipLaunchKernelGGL(dispatch_small_kernel<FS2MOE_MAX_TOP_K>, dim3(1), dim3(kDispTok), lds, s,
+                       topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm, topk_w,
+                       row_w);
+  return check_launch("dispatch_small (row weights)");
+}
+
 extern "C" int64_t fs2moe_dispatch_workspace_bytes(int32_t T, int32_t K, int32_t E) {
   if (T < 0 || K < 1 || E < 1) return -1;
   const int64_t nb = (T + kDispTok - 1) / kDispTok;
@@ -559,12 +579,15 @@ extern "C" int fs2moe_dispatch(const int32_t* topk_idx, const float* topk_w, con
   const bool small = nb == 1 && E <= kDispTok;
   if (small && xe == nullptr) {
     const size_t lds = dispatch_small_lds_words(E) * sizeof(uint32_t);
+    const float* no_w = nullptr;
+    float* no_row_w = nullptr;
     if (K <= 16)
       hipLaunchKernelGGL(dispatch_small_kernel<16>, dim3(1), dim3(kDispTok), lds, s, topk_idx, T, K,
-                         E, tile_m, max_rows, counts, offsets, perm, inv_perm);
+                         E, tile_m, max_rows, counts, offsets, perm, inv_perm, no_w, no_row_w);
     else
       hipLaunchKernelGGL(dispatch_small_kernel<FS2MOE_MAX_TOP_K>, dim3(1), dim3(kDispTok), lds, s,
-                         topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm);
+                         topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm, no_w,
+                         no_row_w);
     return check_launch("dispatch_small");
   }
   if (small) {

@@ -20,12 +20,14 @@ __host__ __device__ inline size_t dispatch_small_lds_words(int E) {
 // KCAP: a compile-time bound on K.  E <= 256 (a thread per expert in the scan).
 // Called by every thread of a block of `nthreads` >= 256 threads (a multiple of 64); threads 0..255
 // are the tokens' threads, the others only help with the loops over LDS and pass the barriers.
-// topk_idx may have been written by this block before a barrier.
+// topk_idx (and topk_w, read only when row_w is given) may have been written by this block before a
+// barrier.
 template <int KCAP>
 __device__ __forceinline__ void dispatch_small_block(
     const int32_t* topk_idx, int T, int K, int E, int tile_m, int64_t max_rows, int32_t* counts,
     int32_t* offsets, int32_t* perm, int32_t* inv_perm, uint32_t* s_mem, int32_t* s_wave_tot,
-    int tid, int nthreads, bool write = true) {
+    int tid, int nthreads, bool write = true, const float* topk_w = nullptr,
+    float* row_w = nullptr) {
   uint32_t* s_bits = s_mem;                    // [E][kDispWords] membership bitmaps
   uint32_t* s_pref = s_mem + E * kDispWords;   // [E][kDispWords] members in the words below
   int32_t* s_off = reinterpret_cast<int32_t*>(s_pref + E * kDispWords);  // [E + 1]
@@ -101,6 +103,8 @@ __device__ __forceinline__ void dispatch_small_block(
         const int row = s_off[ek[k]] + (int)(s_pref[i] + __popc(s_bits[i] & (bit - 1u)));
         inv_perm[p] = row;
         perm[row] = t;
+        // (for kernels that scale a row by its routing weight while they read it through perm)
+        if (row_w != nullptr) row_w[row] = topk_w[p];
       }
     }
   }

@@ -415,9 +415,10 @@ static bool gemv_applies(int act_dtype, int D, int F, const Groups& g, int rows_
 }
 
 template <int R>
-static int launch_gemv_pair_r(const void* x, const int32_t* row_map, const Groups& g,
-                              const void* w_gate, const void* w_up, const void* w_down, int D, int F,
-                              void* h, void* y, hipStream_t stream) {
+static int launch_gemv_pair_r(const void* x, const int32_t* row_map, const float* row_w,
+                              const Groups& g, const void* w_gate, const void* w_up,
+                              const void* w_down, int D, int F, void* h, void* y,
+                              hipStream_t stream) {
   using namespace gemv;
   auto k1 = glu_gemv_bf16_kernel<true, R>;
   auto k2 = glu_gemv_bf16_kernel<false, R>;
@@ -434,13 +435,14 @@ static int launch_gemv_pair_r(const void* x, const int32_t* row_map, const Group
   }
   const uint16_t* xp = static_cast<const uint16_t*>(x);
   hipLaunchKernelGGL(k1, dim3((unsigned)((F + COLS - 1) / COLS), (unsigned)g.E), dim3(threads(R)),
-                     (size_t)R * D * 2, stream, xp, row_map, D, static_cast<const uint16_t*>(w_gate),
+                     (size_t)R * D * 2, stream, xp, row_map, row_w, D, static_cast<const uint16_t*>(w_gate),
                      static_cast<const uint16_t*>(w_up), static_cast<uint16_t*>(h), F, D, F,
                      g.counts, g.offsets);
   if (int rc = check_launch("glu_gemv_bf16<gate,up>")) return rc;
   hipLaunchKernelGGL(k2, dim3((unsigned)((D + COLS - 1) / COLS), (unsigned)g.E), dim3(threads(R)),
                      (size_t)R * F * 2, stream, static_cast<const uint16_t*>(h),
-                     static_cast<const int32_t*>(nullptr), F, static_cast<const uint16_t*>(w_down),
+                     static_cast<const int32_t*>(nullptr), static_cast<const float*>(nullptr), F,
+                     static_cast<const uint16_t*>(w_down),
                      static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(y), D, F, D,
                      g.counts, g.offsets);
   return check_launch("glu_gemv_bf16<down>");
@@ -467,9 +469,10 @@ static int gemv16_rows(int D, int F, int rows_hint) {
 }
 
 template <int XR>
-static int launch_gemv16_pair(const void* x, const int32_t* row_map, const Groups& g,
-                              const void* w_gate, const void* w_up, const void* w_down, int D, int F,
-                              void* h, void* y, hipStream_t stream) {
+static int launch_gemv16_pair(const void* x, const int32_t* row_map, const float* row_w,
+                              const Groups& g, const void* w_gate, const void* w_up,
+                              const void* w_down, int D, int F, void* h, void* y,
+                              hipStream_t stream) {
   using namespace gemv16;
   auto k1 = glu_gemv16_bf16_kernel<true, XR>;
   auto k2 = glu_gemv16_bf16_kernel<false, XR>;
@@ -485,13 +488,14 @@ static int launch_gemv16_pair(const void* x, const int32_t* row_map, const Group
     attr_set = true;
   }
   hipLaunchKernelGGL(k1, dim3((unsigned)((F + COLS - 1) / COLS), (unsigned)g.E), dim3(THREADS),
-                     lds_bytes(D, XR, true), stream, static_cast<const uint16_t*>(x), row_map, D,
+                     lds_bytes(D, XR, true), stream, static_cast<const uint16_t*>(x), row_map, row_w, D,
                      static_cast<const uint16_t*>(w_gate), static_cast<const uint16_t*>(w_up),
                      static_cast<uint16_t*>(h), F, D, F, g.counts, g.offsets);
   if (int rc = check_launch("glu_gemv16_bf16<gate,up>")) return rc;
   hipLaunchKernelGGL(k2, dim3((unsigned)((D + COLS - 1) / COLS), (unsigned)g.E), dim3(THREADS),
                      lds_bytes(F, XR, false), stream, static_cast<const uint16_t*>(h),
-                     static_cast<const int32_t*>(nullptr), F, static_cast<const uint16_t*>(w_down),
+                     static_cast<const int32_t*>(nullptr), static_cast<const float*>(nullptr), F,
+                     static_cast<const uint16_t*>(w_down),
                      static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(y), D, F, D,
                      g.counts, g.offsets);
   return check_launch("glu_gemv16_bf16<down>");
@@ -521,7 +525,8 @@ static int launch_dense_gemv_pair(const void* x, int T, const void* w_gate, cons
 template <int BLAYOUT>
 static int launch_glu(const void* x, const int32_t* row_map, const Groups& g, int64_t rows_bound,
                       const void* w_gate, const void* w_up, const void* w_down, int D, int F,
-                      int act_dtype, void* h, void* y, hipStream_t stream, int rows_hint = 0) {
+                      int act_dtype, void* h, void* y, hipStream_t stream, int rows_hint = 0,
+                      const float* row_w = nullptr) {
   const int groups = g.counts ? g.E : 0;
   if constexpr (BLAYOUT == FS2MOE_W_OUT_IN) {
     if (row_map == nullptr && dense_gemv_applies(act_dtype, g, rows_bound))
@@ -529,15 +534,19 @@ static int launch_glu(const void* x, const int32_t* row_map, const Groups& g, in
   }
   if constexpr (BLAYOUT == FS2MOE_W_IN_OUT) {
     if (gemv_applies(act_dtype, D, F, g, rows_hint)) {
-      if (rows_hint <= 1) return launch_gemv_pair_r<1>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
-      if (rows_hint <= 2) return launch_gemv_pair_r<2>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
-      return launch_gemv_pair_r<4>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
+      if (rows_hint <= 1) return launch_gemv_pair_r<1>(x, row_map, row_w, g, w_gate, w_up, w_down, D, F, h, y, stream);
+      if (rows_hint <= 2) return launch_gemv_pair_r<2>(x, row_map, row_w, g, w_gate, w_up, w_down, D, F, h, y, stream);
+      return launch_gemv_pair_r<4>(x, row_map, row_w, g, w_gate, w_up, w_down, D, F, h, y, stream);
     }
     if (gemv16_applies(act_dtype, D, F, g, rows_hint)) {
       if (gemv16_rows(D, F, rows_hint) == 8)
-        return launch_gemv16_pair<8>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
-      return launch_gemv16_pair<16>(x, row_map, g, w_gate, w_up, w_down, D, F, h, y, stream);
+        return launch_gemv16_pair<8>(x, row_map, row_w, g, w_gate, w_up, w_down, D, F, h, y, stream);
+      return launch_gemv16_pair<16>(x, row_map, row_w, g, w_gate, w_up, w_down, D, F, h, y, stream);
     }
+  }
+  if (row_w != nullptr) {
+    set_error("experts: internal: row weights given to kernels that do not scale rows");
+    return FS2MOE_ERR_UNSUPPORTED;
   }
   if (dma_path_applies(act_dtype, D, F) && dma_offsets_fit(rows_bound, D, F))
     return launch_dma_pair<BLAYOUT>(x, row_map, g, rows_bound, w_gate, w_up, w_down, nullptr, nullptr,
@@ -634,9 +643,12 @@ static int grouped_swiglu_impl(const void* xe, const int32_t* row_map, const int
                                const void* w_down, const float* s_gate, const float* s_up,
                                const float* s_down, int32_t E, int32_t D, int32_t F,
                                int64_t max_rows, int32_t act_dtype, int32_t w_dtype, void* h,
-                               void* ye, int32_t rows_hint, void* stream) {
+                               void* ye, int32_t rows_hint, void* stream,
+                               const float* row_w = nullptr) {
   FS2_REQUIRE(xe && counts && offsets && w_gate && w_up && w_down && h && ye,
               "grouped_swiglu: null pointer");
+  FS2_REQUIRE(row_w == nullptr || w_dtype == FS2MOE_BF16,
+              "grouped_swiglu: internal: row weights go with bf16 weights");
   FS2_REQUIRE(rows_hint >= 0, "grouped_swiglu: rows_per_expert=%d", rows_hint);
   FS2_REQUIRE(E >= 1 && E <= FS2MOE_MAX_EXPERTS, "grouped_swiglu: E=%d outside [1, %d]", E,
               FS2MOE_MAX_EXPERTS);
@@ -726,7 +738,29 @@ static int grouped_swiglu_impl(const void* xe, const int32_t* row_map, const int
   if (max_rows == 0) return FS2MOE_OK;
   Groups g{counts, offsets, E, 0};
   return launch_glu<FS2MOE_W_IN_OUT>(xe, row_map, g, max_rows, w_gate, w_up, w_down, D, F, act_dtype,
-                                     h, ye, static_cast<hipStream_t>(stream), rows_hint);
+                                     h, ye, static_cast<hipStream_t>(stream), rows_hint, row_w);
+}
+
+bool fs2moe::swiglu_streams_rows(int32_t act_dtype, int32_t w_dtype, int32_t D, int32_t F, int32_t E,
+                                 int32_t rows_per_expert) {
+  if (act_dtype != FS2MOE_BF16 || w_dtype != FS2MOE_BF16 || D < 8 || F < 8 || D % 8 || F % 8) return false;
+  static const int32_t some = 0;  // (the predicates only ask whether the groups have counts)
+  const Groups g{&some, &some, E, 0};
+  return gemv_applies(act_dtype, D, F, g, rows_per_expert) || gemv16_applies(act_dtype, D, F, g, rows_per_expert);
+}
+
+int fs2moe::grouped_swiglu_scaled_rows(const void* x, const int32_t* row_map, const float* row_w,
+                                       const int32_t* counts, const int32_t* offsets,
+                                       const void* w_gate, const void* w_up, const void* w_down,
+                                       int32_t E, int32_t D, int32_t F, int64_t max_rows, void* h,
+                                       void* ye, int32_t rows_per_expert, void* stream) {
+  FS2_REQUIRE(row_map && row_w, "grouped_swiglu: null pointer");
+  FS2_REQUIRE(swiglu_streams_rows(FS2MOE_BF16, FS2MOE_BF16, D, F, E, rows_per_expert),
+              "grouped_swiglu: internal: D=%d F=%d E=%d with %d rows an expert do not stream", D, F, E,
+              rows_per_expert);
+  return grouped_swiglu_impl(x, row_map, counts, offsets, w_gate, w_up, w_down, nullptr, nullptr,
+                             nullptr, E, D, F, max_rows, FS2MOE_BF16, FS2MOE_BF16, h, ye,
+                             rows_per_expert, stream, row_w);
 }
 
 extern "C" int fs2moe_grouped_swiglu(const void* xe, const int32_t* row_map, const int32_t* counts,

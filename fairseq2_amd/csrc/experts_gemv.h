@@ -60,11 +60,14 @@ __device__ __forceinline__ int nth_active_expert(const int32_t* __restrict__ cou
 }
 
 // DUAL: C[r, n] = SiLU(A[r] . B0[:, n]) * (A[r] . B1[:, n]); else C[r, n] = A[r] . B0[:, n].
-// A rows are read through row_map when it is given (row r of the expert is A[row_map[offset + r]]).
+// A rows are read through row_map when it is given (row r of the expert is A[row_map[offset + r]]),
+// and multiplied by row_w[offset + r] on the way into LDS when that is given (rounded to bf16: the
+// bits dispatch's scaled row copy would have held).
 // grid: (ceil(N / 64), E).  K a multiple of 4, N a multiple of 8.
 template <bool DUAL, int R>
 __global__ __launch_bounds__(gemv::threads(R)) void glu_gemv_bf16_kernel(
-    const uint16_t* __restrict__ A, const int32_t* __restrict__ row_map, int lda,
+    const uint16_t* __restrict__ A, const int32_t* __restrict__ row_map,
+    const float* __restrict__ row_w, int lda,
     const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1, uint16_t* __restrict__ C,
     int ldc, int K, int N, const int32_t* __restrict__ counts,
     const int32_t* __restrict__ offsets) {
@@ -99,6 +102,10 @@ __global__ __launch_bounds__(gemv::threads(R)) void glu_gemv_bf16_kernel(
         const int row = off + r0 + r;
         const size_t src = (size_t)(row_map != nullptr ? row_map[row] : row) * lda;
         v = *reinterpret_cast<const u32x2*>(A + src + 4 * c);
+        if (row_w != nullptr) {
+          const float w = row_w[row];
+          v = u32x2{scale_bf16x2(v[0], w), scale_bf16x2(v[1], w)};
+        }
       }
       *reinterpret_cast<u32x2*>(xs + (size_t)r * K + 4 * c) = v;
     }
@@ -251,7 +258,8 @@ inline bool offsets_fit(int D, int F) { return (int64_t)D * F * 2 <= 0xffffffffl
 // per CU ran as a full round and a quarter-full one: 4 us of 75 at 8 tokens.)
 template <bool DUAL, int XR>
 __global__ __launch_bounds__(gemv16::THREADS, DUAL ? 2 : 4) void glu_gemv16_bf16_kernel(
-    const uint16_t* __restrict__ A, const int32_t* __restrict__ row_map, int lda,
+    const uint16_t* __restrict__ A, const int32_t* __restrict__ row_map,
+    const float* __restrict__ row_w, int lda,
     const uint16_t* __restrict__ B0, const uint16_t* __restrict__ B1, uint16_t* __restrict__ C,
     int ldc, int K, int N, const int32_t* __restrict__ counts,
     const int32_t* __restrict__ offsets) {
@@ -292,9 +300,11 @@ __global__ __launch_bounds__(gemv16::THREADS, DUAL ? 2 : 4) void glu_gemv16_bf16
       const int kchunks = K / 8;
       const bool has = r0 + r < cnt;
       size_t src = 0;
+      float w = 1.f;
       if (has) {
         const int row = off + r0 + r;
         src = (size_t)(row_map != nullptr ? row_map[row] : row) * lda;
+        if (row_w != nullptr) w = row_w[row];
       }
       for (int cb = c0; cb < kchunks; cb += TPR * INFLIGHT) {
         u32x4 v[INFLIGHT];
@@ -308,6 +318,9 @@ __global__ __launch_bounds__(gemv16::THREADS, DUAL ? 2 : 4) void glu_gemv16_bf16
           const int c = cb + u * TPR;
           if (c >= kchunks) continue;
           if (!has) v[u] = u32x4{0u, 0u, 0u, 0u};
+          if (row_w != nullptr)  // (block-uniform; as dispatch's scaled copy rounds)
+            v[u] = u32x4{scale_bf16x2(v[u][0], w), scale_bf16x2(v[u][1], w), scale_bf16x2(v[u][2], w),
+                         scale_bf16x2(v[u][3], w)};
           u32x2* dst = reinterpret_cast<u32x2*>(xs + (size_t)r * ldx + 8 * c);  // 8-byte aligned
           dst[0] = u32x2{v[u][0], v[u][1]};
           dst[1] = u32x2{v[u][2], v[u][3]};

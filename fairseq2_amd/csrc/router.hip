@@ -816,7 +816,7 @@ template <int J>
 __global__ __launch_bounds__(kFinishDispatchThreads) void router_finish_dispatch_kernel(
     const float* __restrict__ partial, int slices, const float* __restrict__ bias, int T, int E,
     int K, int score_fn, int renorm, int32_t* topk_idx, float* topk_w, int tile_m, int64_t max_rows,
-    int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv_perm) {
+    int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv_perm, float* row_w) {
   extern __shared__ uint32_t s_mem[];
   __shared__ int32_t s_wave_tot[4];
   const int lane = lane_id();
@@ -843,7 +843,7 @@ __global__ __launch_bounds__(kFinishDispatchThreads) void router_finish_dispatch
   __syncthreads();  // the tokens' experts are written and visible to the block
   // (the host sends K > 16 through router_finish_kernel and the dispatch kernels instead)
   dispatch_small_block<16>(topk_idx, T, K, E, tile_m, max_rows, counts, offsets, perm, inv_perm,
-                           s_mem, s_wave_tot, threadIdx.x, kFinishDispatchThreads);
+                           s_mem, s_wave_tot, threadIdx.x, kFinishDispatchThreads, true, topk_w, row_w);
 }
 
 // ------------------------------------------------------------------------------------ f32 / MFMA
@@ -1259,7 +1259,7 @@ static int router_entry(const void* x, const void* norm_w, float norm_eps, void*
                        dim3(kFinishDispatchThreads), dlds, s,                                     \
                        partial, slices, bias, T, E, K, score_fn, renormalize, topk_idx, topk_w,   \
                        disp->tile_m, disp->max_rows, disp->counts, disp->offsets, disp->perm,     \
-                       disp->inv_perm);                                                           \
+                       disp->inv_perm, disp->row_w);                                              \
     break;
         switch (j) {
           FS2_FINISH_CASE(1)

@@ -86,8 +86,10 @@ def test_ragged_shapes_and_single_tokens(gpu_device, shape):
 def test_decode_steps_with_a_shared_expert(gpu_device, tokens, mode):
     """The token counts at which routed and shared experts stream their weights (1-4 rows on the
     vector ALUs, 5-16 on the matrix pipe; 17: the GEMM tiles), in the reference's routing mode (rows
-    copied and scaled by dispatch) and in softmax mode (rows read through the permutation, dispatch
-    inside the router's second kernel): against the oracle, and single call against stages."""
+    copied and scaled by dispatch in the stages; in the single call up to 16 tokens read through the
+    permutation and scaled by the expert kernels) and in softmax mode (rows read through the
+    permutation, dispatch inside the router's second kernel): against the oracle, and single call
+    against stages."""
     _say("decode step", tokens, mode)
     rm = W.RoutingMode("sigmoid", False, "input") if mode == "reference" else W.RoutingMode("softmax", True, "output")
     spec = W.small_spec(tokens=tokens, model_dim=1024, num_experts=16, top_k=2, inner_dim=320, dtype="bf16",
@@ -101,6 +103,32 @@ def test_decode_steps_with_a_shared_expert(gpu_device, tokens, mode):
         single = m(x)  # (out came from the stages)
     torch.cuda.synchronize()
     assert torch.equal(single, out)
+
+
+@pytest.mark.parametrize("tokens", [1, 3, 4, 9, 16])
+@pytest.mark.parametrize("experts,top_k", [(24, 3), (12, 5), (8, 8)])
+def test_decode_steps_in_the_reference_mode_without_a_row_copy(gpu_device, tokens, experts, top_k):
+    """Up to 16 bf16 tokens in the reference's routing mode: the single call makes no scaled copy of
+    the rows, the streaming expert kernels multiply each row by its routing weight as they stage it
+    (the weights in expert-row order written by the dispatch, which with a multiple of 8 experts runs
+    inside the router's second kernel and otherwise as one block of its own).  Same bits as the
+    stages with the copy, with and without the residual; and the oracle."""
+    _say("decode step, reference mode", tokens, experts, top_k)
+    spec = W.small_spec(tokens=tokens, model_dim=512, num_experts=experts, top_k=top_k, inner_dim=192, dtype="bf16",
+                        shared=False, zipf_s=1.1, mode=W.RoutingMode("sigmoid", False, "input"), seed=70 + tokens)
+    wl = W.make_workload_from_spec(spec)
+    _, idx, _ = oracle_routing(wl)
+    ref = oracle_forward(wl, idx, 16, dtype=torch.float64)
+    m, x, out, *_ = _run(wl, gpu_device)  # (the stages)
+    assert_output_close(out, ref.out, "bf16")
+    res = torch.randn(x.shape, generator=torch.Generator().manual_seed(tokens)).bfloat16().to(gpu_device)
+    with torch.no_grad():
+        single = m(x)
+        single_res = m(x, residual=res)
+        staged_res = m._stages(x.reshape(-1, 512), res.reshape(-1, 512))[0].view(x.shape)
+    torch.cuda.synchronize()
+    assert torch.equal(single, out)
+    assert torch.equal(single_res, staged_res)
 
 
 def test_empty_input(gpu_device):
