@@ -422,9 +422,12 @@ static int launch_gemv_pair_r(const void* x, const int32_t* row_map, const float
   using namespace gemv;
   auto k1 = glu_gemv_bf16_kernel<true, R>;
   auto k2 = glu_gemv_bf16_kernel<false, R>;
+  auto k2d = glu_gemv_bf16_kernel<false, R, true>;  // more loads in flight over a long K
   static bool attr_set = false;  // benign race: setting the attribute is idempotent
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(k1),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS_BYTES) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(k2d),
                             hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS_BYTES) != hipSuccess ||
         hipFuncSetAttribute(reinterpret_cast<const void*>(k2),
                             hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS_BYTES) != hipSuccess) {
@@ -439,8 +442,8 @@ static int launch_gemv_pair_r(const void* x, const int32_t* row_map, const float
                      static_cast<const uint16_t*>(w_up), static_cast<uint16_t*>(h), F, D, F,
                      g.counts, g.offsets);
   if (int rc = check_launch("glu_gemv_bf16<gate,up>")) return rc;
-  hipLaunchKernelGGL(k2, dim3((unsigned)((D + COLS - 1) / COLS), (unsigned)g.E), dim3(threads(R)),
-                     (size_t)R * F * 2, stream, static_cast<const uint16_t*>(h),
+  hipLaunchKernelGGL(deep_applies(F, R) ? k2d : k2, dim3((unsigned)((D + COLS - 1) / COLS), (unsigned)g.E),
+                     dim3(threads(R)), (size_t)R * F * 2, stream, static_cast<const uint16_t*>(h),
                      static_cast<const int32_t*>(nullptr), static_cast<const float*>(nullptr), F,
                      static_cast<const uint16_t*>(w_down),
                      static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(y), D, F, D,

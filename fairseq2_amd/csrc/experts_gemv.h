@@ -30,6 +30,14 @@ constexpr int waves(int R) { return 8; }
 constexpr int threads(int R) { return 64 * waves(R); }
 constexpr int MAX_LDS_BYTES = 144 * 1024;  // (160 KB less the kernel's own partial sums, 16 KB at most)
 inline bool fits(int K, int R) { return (int64_t)K * R * 2 <= MAX_LDS_BYTES; }
+// Steps of K (256 rows a block) whose loads a wave issues before it multiplies any: 4 with one or
+// two rows, 2 with four (registers).  DEEP: 8, for the single product with one or two rows over a
+// long K, where a block is a chain of K / 256 / U round trips (Mixtral's down projection, K 14336:
+// the layer at one token 225 -> 178 us, at two 286 -> 251; a short K would only issue loads that it
+// then masks: Qwen3's K of 768 is three steps, and two tokens took 54 instead of 48 us with 8).
+// The sums do not depend on it: a lane adds its products in the same order.
+constexpr int steps_in_flight(bool dual, int R, bool deep) { return R > 2 ? 2 : (deep && !dual) ? 8 : 4; }
+inline bool deep_applies(int K, int R) { return R <= 2 && K >= 4096; }
 }  // namespace gemv
 
 // The n-th expert that has rows, -1 when there are fewer (wave-uniform; every wave works it out for
@@ -64,7 +72,7 @@ __device__ __forceinline__ int nth_active_expert(const int32_t* __restrict__ cou
 // and multiplied by row_w[offset + r] on the way into LDS when that is given (rounded to bf16: the
 // bits dispatch's scaled row copy would have held).
 // grid: (ceil(N / 64), E).  K a multiple of 4, N a multiple of 8.
-template <bool DUAL, int R>
+template <bool DUAL, int R, bool DEEP = false>
 __global__ __launch_bounds__(gemv::threads(R)) void glu_gemv_bf16_kernel(
     const uint16_t* __restrict__ A, const int32_t* __restrict__ row_map,
     const float* __restrict__ row_w, int lda,
@@ -123,7 +131,7 @@ __global__ __launch_bounds__(gemv::threads(R)) void glu_gemv_bf16_kernel(
         for (int c = 0; c < 8; ++c) acc[m][r][c] = 0.f;
     // U steps of K per iteration, all their loads issued before any arithmetic: a step is one round
     // trip to memory and little else, so the steps' round trips overlap
-    constexpr int U = R <= 2 ? 4 : 2;
+    constexpr int U = gemv::steps_in_flight(DUAL, R, DEEP);
     for (int kb0 = 0; kb0 < K; kb0 += U * KSTEP) {
       u32x4 wvu[U][M][4];
 #pragma unroll

@@ -419,6 +419,8 @@ def test_grouped_swiglu_matches_oracle(gpu_device, dtype, rows_per_expert, d, f)
         (4, [9, 4, 13, 0, 1], 128, 64),               # counts above the bound: walked again, still right
         (4, [4, 2], 8192, 64),
         (4, [4, 1], 18432, 64),                       # the longest K whose four rows fit LDS
+        (1, [1, 0, 1], 128, 4096),                    # a long inner dimension: the second product keeps
+        (2, [2, 1, 0, 2], 64, 4352),                  # eight steps of loads in flight (4352: 17 steps)
         # 5 to 16 rows: the same stream with the arithmetic on the matrix pipe
         (16, [16, 9, 0, 12, 1, 5], 2048, 768),       # the Qwen3 shape
         (12, [12, 3, 7], 72, 40),                     # K and N off the kernel's steps
