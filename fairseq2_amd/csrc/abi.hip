@@ -1,6 +1,7 @@
 // Library-wide pieces of the C ABI: version, thread-local error text, launch checking.
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 
 #include "common.h"
 
@@ -115,9 +116,48 @@ extern "C" int64_t fs2moe_forward_norm_workspace_bytes(int32_t T, int32_t D, int
 
 namespace {
 
+// A stream of the library's own per device, for the shared expert of a decode step.  The shared
+// expert depends on the rows only, and with a handful of tokens the routed path (the router's two
+// small kernels, the dispatch, one or a few experts' weight streams) leaves most of the chip idle
+// while it runs: the shared expert's two kernels go onto this stream, forked from the caller's
+// stream by an event and joined back by another before the combine, so a caller sees one stream's
+// worth of ordering (and a capturing stream captures both branches).  Default priority, created
+// on the first use on a device and kept; the events are reused, which is why the record-and-wait
+// pairs are taken under a lock: between one thread's record and its wait another thread's
+// record of the same event would replace what is waited for.
+struct SideStream {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+  bool tried = false;
+};
+constexpr int kSideDevices = 64;
+SideStream g_side[kSideDevices];
+std::mutex g_side_mu;
+
+// null: no such stream on this device (creation failed once); the caller then runs everything on
+// its own stream.
+SideStream* side_stream() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSideDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_side_mu);
+  SideStream& s = g_side[dev];
+  if (!s.tried) {
+    s.tried = true;
+    if (hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&s.join, hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();  // the failure is handled here: nothing for the next call to find
+      s.stream = nullptr;
+    }
+  }
+  return s.stream != nullptr ? &s : nullptr;
+}
+
 // normed: the rows are RMS-normalised on the way into the router (norm_weight may be null), and
 // every stage reads the normalised copy in the workspace.
-int forward_impl(bool normed, const void* x_in, const void* norm_weight, float norm_eps,
+// may_fork: the shared expert of a few tokens may run on the library's side stream (not for the
+// entry point that must create nothing).
+int forward_impl(bool may_fork, bool normed, const void* x_in, const void* norm_weight, float norm_eps,
                  const void* residual, const void* router, const float* router_bias,
                  const void* w_gate, const void* w_up, const void* w_down, const float* s_gate,
                  const float* s_up, const float* s_down, const void* shared_gate,
@@ -173,53 +213,98 @@ int forward_impl(bool normed, const void* x_in, const void* norm_weight, float n
                                          act_dtype, !fused && !act_q && !scaled_stream, normed, act_q,
                                          scaled_stream);
   FS2_REQUIRE(b.total <= need, "forward: internal: the buffers do not fit the workspace");
-  // (with a few tokens and no rows to copy the router's kernel dispatches as well)
-  fs2moe::DispatchAfterRouter disp = {tile_m,     b.max_rows, b.counts,        b.offsets, b.perm,
-                                      b.inv_perm, b.disp_ws,  b.disp_ws_bytes, b.row_w, false};
-  if (int rc = fs2moe::router_then_dispatch(x, normed ? norm_weight : nullptr, normed ? norm_eps : 0.f,
-                                    normed ? b.xn : nullptr, router, router_bias, T, D, E, K,
-                                    act_dtype, score_fn, renormalize, b.topk_idx, b.topk_w,
-                                    b.router_ws, b.router_ws_bytes, b.xe == nullptr ? &disp : nullptr,
-                                    stream))
-    return rc;
-  if (normed) x = b.xn;
-  if (!disp.done) {
-    if (scaled_stream) {
-      if (int rc = fs2moe::dispatch_with_row_weights(b.topk_idx, b.topk_w, T, K, E, tile_m, b.max_rows,
-                                                     b.counts, b.offsets, b.perm, b.inv_perm, b.row_w,
-                                                     stream))
-        return rc;
-    } else if (int rc = fs2moe_dispatch(b.topk_idx, b.topk_w, x, T, K, E, D, tile_m, act_dtype,
-                                        scale_input, b.max_rows, b.counts, b.offsets, b.perm,
-                                        b.inv_perm, b.xe, b.disp_ws, b.disp_ws_bytes, stream)) {
-      return rc;
+  // The shared expert's output is the row the routed outputs are added onto (moe.py:143-150).  With
+  // at most 16 tokens it runs beside the routed path (see SideStream): from the start when it
+  // reads the caller's rows, after the router when it reads the rows the router normalises.
+  SideStream* side = (shared && may_fork && T <= 16) ? side_stream() : nullptr;
+  const bool beside = side != nullptr && side->stream != static_cast<hipStream_t>(stream);
+  auto shared_on = [&](void* s, const void* rows) {
+    return fs2moe_dense_swiglu(rows, shared_gate, shared_up, shared_down, T, D, F_shared, act_dtype,
+                               b.shared_h, out, s);
+  };
+  auto shared_beside = [&]() -> int {
+    hipStream_t main = static_cast<hipStream_t>(stream);
+    {
+      std::lock_guard<std::mutex> lock(g_side_mu);
+      if (hipEventRecord(side->fork, main) != hipSuccess ||
+          hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess) {
+        fs2moe::set_error("forward: cannot fork the shared expert's stream: %s",
+                          hipGetErrorString(hipGetLastError()));
+        return FS2MOE_ERR_LAUNCH;
+      }
     }
+    return shared_on(side->stream, normed ? b.xn : x_in);
+  };
+  // the caller's stream goes on only when the side stream has come this far (called once the
+  // routed experts are on their way, in front of the combine; and on every way out after a fork,
+  // so that the side stream never stays forked from a capturing stream)
+  auto shared_joins = [&]() -> int {
+    std::lock_guard<std::mutex> lock(g_side_mu);
+    if (hipEventRecord(side->join, side->stream) != hipSuccess ||
+        hipStreamWaitEvent(static_cast<hipStream_t>(stream), side->join, 0) != hipSuccess) {
+      fs2moe::set_error("forward: cannot join the shared expert's stream: %s",
+                        hipGetErrorString(hipGetLastError()));
+      return FS2MOE_ERR_LAUNCH;
+    }
+    return FS2MOE_OK;
+  };
+  bool forked = false;
+  // router, dispatch and the routed experts, with the shared expert forked off on the way
+  auto routed_path = [&]() -> int {
+    if (beside && !normed) {
+      forked = true;
+      if (int rc = shared_beside()) return rc;
+    }
+    // (with a few tokens and no rows to copy the router's kernel dispatches as well)
+    fs2moe::DispatchAfterRouter disp = {tile_m,     b.max_rows, b.counts,        b.offsets, b.perm,
+                                        b.inv_perm, b.disp_ws,  b.disp_ws_bytes, b.row_w,   false};
+    if (int rc = fs2moe::router_then_dispatch(
+            x, normed ? norm_weight : nullptr, normed ? norm_eps : 0.f, normed ? b.xn : nullptr, router,
+            router_bias, T, D, E, K, act_dtype, score_fn, renormalize, b.topk_idx, b.topk_w, b.router_ws,
+            b.router_ws_bytes, b.xe == nullptr ? &disp : nullptr, stream))
+      return rc;
+    if (normed) x = b.xn;
+    if (beside && normed) {
+      forked = true;
+      if (int rc = shared_beside()) return rc;
+    }
+    if (!disp.done) {
+      if (scaled_stream) {
+        if (int rc = fs2moe::dispatch_with_row_weights(b.topk_idx, b.topk_w, T, K, E, tile_m,
+                                                       b.max_rows, b.counts, b.offsets, b.perm,
+                                                       b.inv_perm, b.row_w, stream))
+          return rc;
+      } else if (int rc = fs2moe_dispatch(b.topk_idx, b.topk_w, x, T, K, E, D, tile_m, act_dtype,
+                                          scale_input, b.max_rows, b.counts, b.offsets, b.perm,
+                                          b.inv_perm, b.xe, b.disp_ws, b.disp_ws_bytes, stream)) {
+        return rc;
+      }
+    }
+    if (act_q) {
+      // the token rows to block-scaled e4m3 once; both products read codes (the first through perm)
+      if (int rc = fs2moe_mx_quantize(x, T, D, b.xq, b.xs, stream)) return rc;
+      return fs2moe_grouped_swiglu_w8a8(b.xq, b.xs, b.perm, b.counts, b.offsets, w_gate, w_up, w_down,
+                                        s_gate, s_up, s_down, E, D, F, T, b.max_rows, b.hq, b.hs, b.ye,
+                                        stream);
+    }
+    if (scaled_stream)
+      return fs2moe::grouped_swiglu_scaled_rows(x, b.perm, b.row_w, b.counts, b.offsets, w_gate, w_up,
+                                                w_down, E, D, F, b.max_rows, b.h, b.ye, T, stream);
+    // (a token takes an expert at most once: with up to 16 tokens no expert has more rows than that)
+    return fs2moe_grouped_swiglu_rows(fused ? x : b.xe, fused ? b.perm : nullptr, b.counts, b.offsets,
+                                      w_gate, w_up, w_down, s_gate, s_up, s_down, E, D, F, b.max_rows,
+                                      act_dtype, w_dtype, b.h, b.ye, T <= 16 ? T : 0, stream);
+  };
+  int rc_routed = routed_path();
+  if (forked) {
+    const int rc_join = shared_joins();
+    if (rc_routed == FS2MOE_OK) rc_routed = rc_join;
   }
-  if (act_q) {
-    // the token rows to block-scaled e4m3 once; both products read codes (the first through perm)
-    if (int rc = fs2moe_mx_quantize(x, T, D, b.xq, b.xs, stream)) return rc;
-    if (int rc = fs2moe_grouped_swiglu_w8a8(b.xq, b.xs, b.perm, b.counts, b.offsets, w_gate, w_up,
-                                            w_down, s_gate, s_up, s_down, E, D, F, T, b.max_rows,
-                                            b.hq, b.hs, b.ye, stream))
-      return rc;
-  } else if (scaled_stream) {
-    if (int rc = fs2moe::grouped_swiglu_scaled_rows(x, b.perm, b.row_w, b.counts, b.offsets, w_gate,
-                                                    w_up, w_down, E, D, F, b.max_rows, b.h, b.ye, T,
-                                                    stream))
-      return rc;
-  } else
-  // (a token takes an expert at most once: with up to 16 tokens no expert has more rows than that)
-  if (int rc = fs2moe_grouped_swiglu_rows(fused ? x : b.xe, fused ? b.perm : nullptr, b.counts,
-                                          b.offsets, w_gate, w_up, w_down, s_gate, s_up, s_down, E,
-                                          D, F, b.max_rows, act_dtype, w_dtype, b.h, b.ye,
-                                          T <= 16 ? T : 0, stream))
-    return rc;
+  if (rc_routed != FS2MOE_OK) return rc_routed;
   const void* base = nullptr;
   if (shared) {
-    // the shared expert's output is the row the routed outputs are added onto (moe.py:143-150)
-    if (int rc = fs2moe_dense_swiglu(x, shared_gate, shared_up, shared_down, T, D, F_shared,
-                                     act_dtype, b.shared_h, out, stream))
-      return rc;
+    if (!beside)
+      if (int rc = shared_on(stream, x)) return rc;
     base = out;
   }
   if (residual != nullptr)
@@ -241,7 +326,7 @@ extern "C" int fs2moe_forward(const void* x, const void* residual, const void* r
                               int32_t w_dtype, int32_t score_fn, int32_t renormalize,
                               int32_t scale_input, void* workspace, int64_t workspace_bytes,
                               void* out, void* stream) {
-  return forward_impl(false, x, nullptr, 0.f, residual, router, router_bias, w_gate, w_up, w_down,
+  return forward_impl(true, false, x, nullptr, 0.f, residual, router, router_bias, w_gate, w_up, w_down,
                       s_gate, s_up, s_down, shared_gate, shared_up, shared_down, T, D, E, K, F,
                       F_shared, tile_m, act_dtype, w_dtype, score_fn, renormalize, scale_input,
                       workspace, workspace_bytes, out, stream);
@@ -258,7 +343,7 @@ extern "C" int fs2moe_forward_norm(const void* x, const void* norm_weight, float
                                    int32_t act_dtype, int32_t w_dtype, int32_t score_fn,
                                    int32_t renormalize, int32_t scale_input, void* workspace,
                                    int64_t workspace_bytes, void* out, void* stream) {
-  return forward_impl(true, x, norm_weight, norm_eps, residual, router, router_bias, w_gate, w_up,
+  return forward_impl(true, true, x, norm_weight, norm_eps, residual, router, router_bias, w_gate, w_up,
                       w_down, s_gate, s_up, s_down, shared_gate, shared_up, shared_down, T, D, E, K,
                       F, F_shared, tile_m, act_dtype, w_dtype, score_fn, renormalize, scale_input,
                       workspace, workspace_bytes, out, stream);
@@ -324,8 +409,9 @@ extern "C" int fs2moe_forward_static(const void* x, const void* residual, const 
   if (ws == nullptr) return FS2MOE_ERR_LAUNCH;
   // Every stage writes what it later reads (nothing in the workspace has to start at zero), so the
   // previous call's contents need no clearing.
-  return fs2moe_forward(x, residual, router, router_bias, w_gate, w_up, w_down, s_gate, s_up,
-                        s_down, shared_gate, shared_up, shared_down, T, D, E, K, F, F_shared,
-                        tile_m, act_dtype, w_dtype, score_fn, renormalize, scale_input, ws,
-                        FS2MOE_STATIC_SCRATCH_BYTES, out, stream);
+  // (everything on the caller's stream: this entry point creates nothing, streams included)
+  return forward_impl(false, false, x, nullptr, 0.f, residual, router, router_bias, w_gate, w_up,
+                      w_down, s_gate, s_up, s_down, shared_gate, shared_up, shared_down, T, D, E, K,
+                      F, F_shared, tile_m, act_dtype, w_dtype, score_fn, renormalize, scale_input, ws,
+                      FS2MOE_STATIC_SCRATCH_BYTES, out, stream);
 }

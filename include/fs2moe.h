@@ -245,6 +245,9 @@ int fs2moe_combine_residual(const void* ye, const int32_t* inv_perm, const int32
  *               0: they multiply the experts' output rows
  *   workspace   at least fs2moe_forward_workspace_bytes(...) bytes, 256-byte aligned
  *   out [T, D] act_dtype (out; must not alias x; may alias residual unless there is a shared expert)
+ * With a shared expert and at most 16 tokens the shared expert's kernels run on a stream of the
+ * library's own, forked from `stream` and joined back to it inside the call (events; under stream
+ * capture both branches are captured): to the caller the call is ordered on `stream` as before.
  */
 int64_t fs2moe_forward_workspace_bytes(int32_t T, int32_t D, int32_t E, int32_t K, int32_t F,
                                        int32_t F_shared, int32_t tile_m, int32_t act_dtype);

@@ -555,7 +555,10 @@ class _RMSNorm:
         (W.RoutingMode("softmax", True, "output"), False, "tokens=1"),
         (W.RoutingMode("softmax", True, "output"), True, "tokens=3"),
         (W.RoutingMode("sigmoid", True, "output"), False, "tokens=4"),
-        (W.RoutingMode("sigmoid", False, "input"), False, "tokens=2"),  # rows are copied: no merged dispatch
+        (W.RoutingMode("sigmoid", False, "input"), False, "tokens=2"),  # rows scaled by the expert kernels
+        # a decode step with a shared expert: its kernels beside the routed path, after the router
+        (W.RoutingMode("sigmoid", False, "input"), True, "tokens=5"),
+        (W.RoutingMode("softmax", True, "output"), True, "tokens=16"),
     ],
 )
 def test_pre_norm_and_residual_in_one_call(gpu_device, dtype, mode, shared, weights):
