@@ -216,7 +216,12 @@ int forward_impl(bool may_fork, bool normed, const void* x_in, const void* norm_
   // The shared expert's output is the row the routed outputs are added onto (moe.py:143-150).  With
   // at most 16 tokens it runs beside the routed path (see SideStream): from the start when it
   // reads the caller's rows, after the router when it reads the rows the router normalises.
-  SideStream* side = (shared && may_fork && T <= 16) ? side_stream() : nullptr;
+  // (forking and joining cost the host four calls, about as long as a whole step of a small layer
+  // takes it to launch: D 2048 / F 4096, 16 experts, one token 53 -> 100 us with them, where D 4096 /
+  // F 8192 goes 137 -> 129 and Scout's D 5120 / F 8192 173 -> 156; so only where the shared expert
+  // streams at least 192 MB of weights)
+  const bool big_shared = (int64_t)3 * D * F_shared * fs2moe::elem_size(act_dtype) >= (192ll << 20);
+  SideStream* side = (shared && may_fork && T <= 16 && big_shared) ? side_stream() : nullptr;
   const bool beside = side != nullptr && side->stream != static_cast<hipStream_t>(stream);
   auto shared_on = [&](void* s, const void* rows) {
     return fs2moe_dense_swiglu(rows, shared_gate, shared_up, shared_down, T, D, F_shared, act_dtype,

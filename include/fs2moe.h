@@ -245,7 +245,7 @@ int fs2moe_combine_residual(const void* ye, const int32_t* inv_perm, const int32
  *               0: they multiply the experts' output rows
  *   workspace   at least fs2moe_forward_workspace_bytes(...) bytes, 256-byte aligned
  *   out [T, D] act_dtype (out; must not alias x; may alias residual unless there is a shared expert)
- * With a shared expert and at most 16 tokens the shared expert's kernels run on a stream of the
+ * With a large shared expert (192 MB of weights or more) and at most 16 tokens its kernels run on a stream of the
  * library's own, forked from `stream` and joined back to it inside the call (events; under stream
  * capture both branches are captured): to the caller the call is ordered on `stream` as before.
  */

@@ -281,7 +281,43 @@ def test_mixtral_8x7b_shape(gpu_device):
 
 
 def test_llama4_scout_shape(gpu_device):
-    _full_size_case("llama4_scout", gpu_device, sample=256)
+    wl, m, x, _, _ = _full_size_case("llama4_scout", gpu_device, sample=256)
+    # Decode steps on the same weights.  At this size the single call runs the shared expert's two
+    # kernels on a stream of the library's own, beside the routed path (the stages run them after it):
+    # same bits, repeatedly, with other work of the caller's stream around the calls; and the oracle
+    # (a token's output does not depend on the other tokens of the batch).
+    d = wl.spec.model_dim
+    _, idx, _ = oracle_routing(wl)
+    rows = x.reshape(-1, d)
+    for t in (1, 5, 16):
+        _say("scout decode", t)
+        xt = rows[:t].contiguous()
+        tok = torch.arange(t)
+        ref = oracle_forward(wl, idx, 16, tokens=tok)
+        with torch.no_grad():
+            staged = m._stages(xt, None)[0]
+            singles = []
+            for _ in range(3):
+                xt.add_(0.0)  # (a kernel of the caller's in front of each call)
+                singles.append(m(xt))
+                singles[-1].add_(0.0)  # (and one behind it, reading the result)
+        torch.cuda.synchronize()
+        for got in singles:
+            assert torch.equal(got, staged)
+        assert_output_close(staged, ref.out.reshape(-1, d)[tok], "bf16", f"scout decode, {t} tokens")
+    # the same step captured: the graph holds both streams' kernels and replays to the eager bits
+    from fairseq2_amd import GraphedForward
+
+    xs = [rows[:5].contiguous(), rows[5:10].contiguous(), rows[10:15].contiguous()]
+    with torch.no_grad():
+        eager = [m(xi).clone() for xi in xs]
+        graphed = GraphedForward(m, xs[0])
+        for rep in range(2):
+            for xi, want in zip(xs, eager):
+                got = graphed(xi).clone()
+                torch.cuda.synchronize()
+                assert torch.equal(got, want), "graph replay differs from the eager result"
+                assert torch.equal(m(xi), want)  # eager work between replays
 
 
 def test_qwen3_prefill_shape_with_fp8_weights(gpu_device):
@@ -556,7 +592,7 @@ class _RMSNorm:
         (W.RoutingMode("softmax", True, "output"), True, "tokens=3"),
         (W.RoutingMode("sigmoid", True, "output"), False, "tokens=4"),
         (W.RoutingMode("sigmoid", False, "input"), False, "tokens=2"),  # rows scaled by the expert kernels
-        # a decode step with a shared expert: its kernels beside the routed path, after the router
+        # decode steps with a shared expert
         (W.RoutingMode("sigmoid", False, "input"), True, "tokens=5"),
         (W.RoutingMode("softmax", True, "output"), True, "tokens=16"),
     ],
